@@ -1,23 +1,29 @@
 // A routed feed-forward (mixture of experts) that never leaves the device, so that a step with
 // one can be recorded as a graph:
 //
-//   ptl_moe_topk      per token: scores = sigmoid(logits) in float32, the ``top`` largest, their
-//                     experts and scores (the score is the weight, with or without a
-//                     renormalisation over the chosen ones); and the sigmoid of extra logit columns
-//                     behind the experts' (a gate of a shared expert)
+//   ptl_moe_topk      per token: scores = sigmoid(logits) or softmax(logits) in float32, the ``top``
+//                     largest (by score plus a per-expert correction, when one is given), their
+//                     experts and scores (the score without the correction is the weight, with or
+//                     without a renormalisation over the chosen ones, times a constant); experts
+//                     from ``real`` on have no matrices and return their input: their pairs get
+//                     expert -1 and their weights are added up per token; and the sigmoid of extra
+//                     logit columns behind the experts' (a gate of a shared expert)
 //   ptl_moe_sort      the (token, choice) pairs ordered by expert: positions, the tiles of
 //                     MOE_TM rows that the products walk, all by one workgroup
 //   ptl_moe_gate_up   per tile: rows gathered from x, the expert's gate and up matrices, and
 //                     the gated activation, written in sorted order. The routing weight scales
 //                     the expert's input (it is applied to both products, which are linear) or
 //                     is left for the output
+//   ptl_moe_up        the same for experts without a gate: act(up(x)), one matrix
 //   ptl_moe_down      per tile: the expert's down matrix on the sorted rows
 //   ptl_moe_combine   per token: the sum of its choices' rows (times the weight when it scales
-//                     the output), plus gate * a shared expert's row
+//                     the output), plus gate * a shared expert's row, plus the token's input times
+//                     the weights of its experts that return their input
+//   ptl_unary_act     an ungated expert's activation on a dense product
 //   ptl_gated_act     the experts' activation on a dense [T, 2I] gate|up product
 //
 // Activation kinds: 0: silu(g) * u;  1: g' = min(g, limit), u' = clamp(u, -limit, limit),
-// g' * sigmoid(1.702 g') * (u' + 1).
+// g' * sigmoid(1.702 g') * (u' + 1). Without a gate: 2: relu(u)^2.
 #include "common.h"
 #include "mfma.h"
 #include <math.h>
@@ -35,23 +41,58 @@ __device__ __forceinline__ float gated_act(int kind, float g, float u, float lim
   return g * sigmoidf_(g) * u;
 }
 
+__device__ __forceinline__ float unary_act(int kind, float u) {
+  (void)kind;                            // (2: the square of relu, the only one so far)
+  const float r = fmaxf(u, 0.f);
+  return r * r;
+}
+
 // One wave a token. Lane l holds the logits of experts l, l + 64, ...
 #define TOPK_PER_LANE 16
+#define SCORE_SIGMOID 0
+#define SCORE_SOFTMAX 1
 __global__ void __launch_bounds__(256)
 moe_topk_kernel(const float* __restrict__ logits, int ld, int T_, int E, int top, int extra,
-                int renormalize, int32_t* __restrict__ idx, float* __restrict__ wgt,
-                float* __restrict__ extra_out) {
+                int renormalize, int score_fn, const float* __restrict__ bias, int real, float renorm_eps,
+                float wscale, int32_t* __restrict__ idx, float* __restrict__ wgt,
+                float* __restrict__ extra_out, float* __restrict__ ident_out) {
   const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
   if (t >= T_) return;
   const float* z = logits + (size_t)t * ld;
-  float v[TOPK_PER_LANE];
+  // v: what the choice goes by; sc: the score that becomes the weight. Sigmoid scores without a
+  // correction are chosen by their logits (the same order, and no ties where the sigmoid saturates).
+  float v[TOPK_PER_LANE], sc[TOPK_PER_LANE];
+  float zmax = -INFINITY;
 #pragma unroll
   for (int i = 0; i < TOPK_PER_LANE; ++i) {
     const int e = lane + 64 * i;
     v[i] = e < E ? z[e] : -INFINITY;
+    zmax = fmaxf(zmax, v[i]);
   }
-  float sum = 0.f;
+  if (score_fn == SCORE_SOFTMAX) {
+    zmax = wave_max(zmax);
+    float den = 0.f;
+#pragma unroll
+    for (int i = 0; i < TOPK_PER_LANE; ++i) {
+      sc[i] = lane + 64 * i < E ? expf(v[i] - zmax) : 0.f;
+      den += sc[i];
+    }
+    den = wave_sum(den);
+#pragma unroll
+    for (int i = 0; i < TOPK_PER_LANE; ++i) sc[i] /= den;
+  } else {
+#pragma unroll
+    for (int i = 0; i < TOPK_PER_LANE; ++i) sc[i] = sigmoidf_(v[i]);
+  }
+  if (score_fn == SCORE_SOFTMAX || bias) {
+#pragma unroll
+    for (int i = 0; i < TOPK_PER_LANE; ++i) {
+      const int e = lane + 64 * i;
+      if (e < E) v[i] = bias ? sc[i] + bias[e] : sc[i];
+    }
+  }
+  float sum = 0.f, ident = 0.f;
   for (int k = 0; k < top; ++k) {
     float best = -INFINITY;
     int at = 0x7fffffff;
@@ -73,32 +114,55 @@ moe_topk_kernel(const float* __restrict__ logits, int ld, int T_, int E, int top
       }
     }
     if (at >= E) at = k;                 // (only when a logit is NaN: the NaN then shows in the output)
+    float mine = 0.f;
 #pragma unroll
     for (int i = 0; i < TOPK_PER_LANE; ++i)
-      if (lane + 64 * i == at) v[i] = -INFINITY;
-    const float s = sigmoidf_(best);
+      if (lane + 64 * i == at) {
+        v[i] = -INFINITY;
+        mine = sc[i];
+      }
+    const float s = __shfl(mine, at & 63, 64);
     sum += s;
     if (lane == 0) {
-      idx[(size_t)t * top + k] = at;
+      idx[(size_t)t * top + k] = at < real ? at : -1;
       wgt[(size_t)t * top + k] = s;
     }
   }
-  if (renormalize && lane == 0)
-    for (int k = 0; k < top; ++k) wgt[(size_t)t * top + k] /= sum;
+  if (lane == 0) {
+    for (int k = 0; k < top; ++k) {
+      float w = wgt[(size_t)t * top + k];
+      if (renormalize || wscale != 1.f) {
+        if (renormalize) w /= sum + renorm_eps;
+        w *= wscale;
+        wgt[(size_t)t * top + k] = w;
+      }
+      if (idx[(size_t)t * top + k] < 0) ident += w;
+    }
+    if (ident_out) ident_out[t] = ident;
+  }
   if (lane < extra) extra_out[(size_t)t * extra + lane] = sigmoidf_(z[E + lane]);
 }
 
+// logits [T, ld]: E router outputs a row, then ``extra`` columns. score_fn: 0 sigmoid, 1 softmax over
+// the E outputs. bias [E] or null: added to the scores for the choice only. real: the first ``real``
+// outputs are experts with matrices, the others return their input (idx -1; ident_out [T], which
+// must be given when real < E, receives the sum of their weights). Weights: the scores, divided by
+// their sum + renorm_eps when ``renormalize``, times wscale.
 extern "C" int ptl_moe_topk(const float* logits, int ld, int T_, int E, int top, int extra, int renormalize,
-                            int32_t* idx, float* wgt, float* extra_out, hipStream_t st) {
+                            int score_fn, const float* bias, int real, float renorm_eps, float wscale,
+                            int32_t* idx, float* wgt, float* extra_out, float* ident_out, hipStream_t st) {
   if (T_ <= 0) return PTL_OK;
   if (E <= 0 || top <= 0 || top > E || E > 64 * TOPK_PER_LANE || extra < 0 || extra > 64 || ld < E + extra ||
-      (extra && !extra_out))
+      (extra && !extra_out) || real < 0 || real > E || (real < E && !ident_out) ||
+      (score_fn != SCORE_SIGMOID && score_fn != SCORE_SOFTMAX))
     return PTL_ERR_ARG;
-  moe_topk_kernel<<<(T_ + 3) / 4, 256, 0, st>>>(logits, ld, T_, E, top, extra, renormalize, idx, wgt, extra_out);
+  moe_topk_kernel<<<(T_ + 3) / 4, 256, 0, st>>>(logits, ld, T_, E, top, extra, renormalize, score_fn, bias, real,
+                                                renorm_eps, wscale, idx, wgt, extra_out, ident_out);
   return ptl_launch_status();
 }
 
-// One workgroup. A = pairs (token, choice). Writes: pos_of[a] (the sorted position of pair a),
+// One workgroup. A = pairs (token, choice). Writes: pos_of[a] (the sorted position of pair a; -1
+// for a pair whose expert is outside 0..E-1 and takes no part in the products),
 // sorted[p] (the pair at position p), expert_end[e] (one past the last position of expert e),
 // and the tile list: tile_expert[i] (-1: no tile), tile_row0[i] for i < max_tiles.
 __global__ void __launch_bounds__(1024)
@@ -140,7 +204,10 @@ moe_sort_kernel(const int32_t* __restrict__ idx, int A, int E, int32_t* __restri
   // to run, the results do not (a row's result does not depend on its place in a tile)
   for (int a = threadIdx.x; a < A; a += 1024) {
     const int e = idx[a];
-    if (e < 0 || e >= E) continue;
+    if (e < 0 || e >= E) {                 // a pair without an expert's matrices
+      pos_of[a] = -1;
+      continue;
+    }
     const int p = start[e] + atomicAdd(&count[e], 1);
     sorted[p] = a;
     pos_of[a] = p;
@@ -164,13 +231,20 @@ extern "C" int ptl_moe_sort(const int32_t* idx, int A, int E, int32_t* pos_of, i
 // MOE_TM sorted rows x 64 result columns a workgroup; the gate|up product keeps two sums an
 // output (gate row n and up row I + n of the expert's [2 I, K] matrix).
 #define MK 16
+// what a product is: the down matrix on the sorted rows; gate|up on rows gathered from x, with
+// the gated activation; up alone on gathered rows, with an activation of one value
+#define MODE_DOWN 0
+#define MODE_GATE_UP 1
+#define MODE_UP 2
 
-template <typename T, bool GATE_UP>
+template <typename T, int MODE>
 __global__ void __launch_bounds__(256)
 moe_gemm_kernel(T* __restrict__ out, long ldo, const T* __restrict__ x, long ldx, const T* __restrict__ w,
                 const int32_t* __restrict__ tile_expert, const int32_t* __restrict__ tile_row0,
                 const int32_t* __restrict__ expert_end, const int32_t* __restrict__ sorted,
                 const float* __restrict__ wgt, int top, int N, int K, int act, float limit) {
+  constexpr bool GATE_UP = MODE == MODE_GATE_UP;
+  constexpr bool GATHER = MODE != MODE_DOWN;
   const int e = tile_expert[blockIdx.y];
   if (e < 0) return;
   const int row0 = tile_row0[blockIdx.y];
@@ -184,7 +258,7 @@ moe_gemm_kernel(T* __restrict__ out, long ldo, const T* __restrict__ x, long ldx
     int r = -1;
     float f = 1.f;
     if (tid < rows) {
-      if (GATE_UP) {
+      if (GATHER) {
         const int a = sorted[row0 + tid];
         r = a / top;
         if (wgt) f = wgt[a];
@@ -248,6 +322,8 @@ moe_gemm_kernel(T* __restrict__ out, long ldo, const T* __restrict__ x, long ldx
       float v;
       if (GATE_UP)
         v = gated_act(act, acc[0][i][j] * f, acc[GATE_UP ? 1 : 0][i][j] * f, limit);
+      else if (MODE == MODE_UP)
+        v = unary_act(act, acc[0][i][j] * f);
       else
         v = acc[0][i][j];
       out[(size_t)(row0 + m) * ldo + n] = from_float<T>(v);
@@ -261,13 +337,15 @@ moe_gemm_kernel(T* __restrict__ out, long ldo, const T* __restrict__ x, long ldx
 // tile of at most 16 rows (nearly every tile of a decode step) is shared by the four waves
 // along K, 32 values in turn, so that four times as many loads of the expert's weights are under
 // way; their partial sums meet in LDS. Taller tiles: a wave owns 16 of the rows.
-template <bool GATE_UP>
+template <int MODE>
 __global__ void __launch_bounds__(256)
 moe_gemm_mfma_kernel(bf16_t* __restrict__ out, long ldo, const bf16_t* __restrict__ x, long ldx,
                      const bf16_t* __restrict__ w, const int32_t* __restrict__ tile_expert,
                      const int32_t* __restrict__ tile_row0, const int32_t* __restrict__ expert_end,
                      const int32_t* __restrict__ sorted, const float* __restrict__ wgt, int top, int N, int K,
                      int act, float limit) {
+  constexpr bool GATE_UP = MODE == MODE_GATE_UP;
+  constexpr bool GATHER = MODE != MODE_DOWN;
   constexpr int G = GATE_UP ? 2 : 1;
   __shared__ float red[3][G * 4][4][64];
   const int e = tile_expert[blockIdx.y];
@@ -285,7 +363,7 @@ moe_gemm_mfma_kernel(bf16_t* __restrict__ out, long ldo, const bf16_t* __restric
   const int mr = min(ln, rows - 1);
   int src = row0 + mr;
   float f = 1.f;
-  if (GATE_UP) {
+  if (GATHER) {
     const int a = sorted[src];
     src = a / top;
     if (wgt) f = wgt[a];
@@ -347,6 +425,8 @@ moe_gemm_mfma_kernel(bf16_t* __restrict__ out, long ldo, const bf16_t* __restric
         float v;
         if (GATE_UP)
           v = gated_act(act, acc[0][j][i] * f, acc[G - 1][j][i] * f, limit);
+        else if (MODE == MODE_UP)
+          v = unary_act(act, acc[0][j][i] * f);
         else
           v = acc[0][j][i];
         out[(size_t)(row0 + ln) * ldo + n] = float_to_bf16(v);
@@ -366,13 +446,15 @@ moe_gemm_mfma_kernel(bf16_t* __restrict__ out, long ldo, const bf16_t* __restric
 #define TB_K 64
 #define TB_BROWS 128
 
-template <bool GATE_UP>
+template <int MODE>
 __global__ void __launch_bounds__(256)
 moe_gemm_tiled_kernel(bf16_t* __restrict__ out, long ldo, const bf16_t* __restrict__ x, long ldx,
                       const bf16_t* __restrict__ w, const int32_t* __restrict__ tile_expert,
                       const int32_t* __restrict__ tile_row0, const int32_t* __restrict__ expert_end,
                       const int32_t* __restrict__ sorted, const float* __restrict__ wgt, int top, int N, int K,
                       int act, float limit) {
+  constexpr bool GATE_UP = MODE == MODE_GATE_UP;
+  constexpr bool GATHER = MODE != MODE_DOWN;
   const int e = tile_expert[blockIdx.y];
   if (e < 0) return;
   __shared__ __attribute__((aligned(1024))) bf16_t As0[64 * TB_K];
@@ -388,7 +470,7 @@ moe_gemm_tiled_kernel(bf16_t* __restrict__ out, long ldo, const bf16_t* __restri
     const int t = min(tid, rows - 1);
     int r;
     float f = 1.f;
-    if (GATE_UP) {
+    if (GATHER) {
       const int a = sorted[row0 + t];
       r = a / top;
       if (wgt) f = wgt[a];
@@ -496,7 +578,7 @@ moe_gemm_tiled_kernel(bf16_t* __restrict__ out, long ldo, const bf16_t* __restri
         const int n = GATE_UP ? n0 + cg * 32 + 16 * j + 4 * lg + q : n0 + cg * 64 + 16 * j + 4 * lg + q;
         if (n >= N) continue;
         const float v = GATE_UP ? gated_act(act, acc[i][j][q] * f, acc[i][GATE_UP ? j + 2 : j][q] * f, limit)
-                                : acc[i][j][q];
+                                : (MODE == MODE_UP ? unary_act(act, acc[i][j][q] * f) : acc[i][j][q]);
         orow[n] = float_to_bf16(v);
       }
   }
@@ -520,23 +602,54 @@ extern "C" int ptl_moe_gate_up(void* out, long ldo, const void* x, long ldx, con
   if (I <= 0 || K <= 0 || top <= 0 || max_tiles > 65535) return PTL_ERR_ARG;
   dim3 grid((I + 63) / 64, max_tiles);
   if (dtype == PTL_DTYPE_F32)
-    moe_gemm_kernel<float, true><<<grid, 256, 0, st>>>((float*)out, ldo, (const float*)x, ldx, (const float*)w,
+    moe_gemm_kernel<float, MODE_GATE_UP><<<grid, 256, 0, st>>>((float*)out, ldo, (const float*)x, ldx, (const float*)w,
                                                        tile_expert, tile_row0, expert_end, sorted, wgt, top, I,
                                                        K, act, limit);
   else if (dtype == PTL_DTYPE_BF16 && mfma_ok(x, ldx, w, K) && pairs >= MOE_TILED_FROM && K % TB_K == 0) {
     dim3 wide((I + TB_BROWS / 2 - 1) / (TB_BROWS / 2), max_tiles);
-    moe_gemm_tiled_kernel<true><<<wide, 256, 0, st>>>((bf16_t*)out, ldo, (const bf16_t*)x, ldx,
+    moe_gemm_tiled_kernel<MODE_GATE_UP><<<wide, 256, 0, st>>>((bf16_t*)out, ldo, (const bf16_t*)x, ldx,
                                                       (const bf16_t*)w, tile_expert, tile_row0, expert_end,
                                                       sorted, wgt, top, I, K, act, limit);
   }
   else if (dtype == PTL_DTYPE_BF16 && mfma_ok(x, ldx, w, K))
-    moe_gemm_mfma_kernel<true><<<grid, 256, 0, st>>>((bf16_t*)out, ldo, (const bf16_t*)x, ldx,
+    moe_gemm_mfma_kernel<MODE_GATE_UP><<<grid, 256, 0, st>>>((bf16_t*)out, ldo, (const bf16_t*)x, ldx,
                                                      (const bf16_t*)w, tile_expert, tile_row0, expert_end,
                                                      sorted, wgt, top, I, K, act, limit);
   else if (dtype == PTL_DTYPE_BF16)
-    moe_gemm_kernel<bf16_t, true><<<grid, 256, 0, st>>>((bf16_t*)out, ldo, (const bf16_t*)x, ldx,
+    moe_gemm_kernel<bf16_t, MODE_GATE_UP><<<grid, 256, 0, st>>>((bf16_t*)out, ldo, (const bf16_t*)x, ldx,
                                                         (const bf16_t*)w, tile_expert, tile_row0, expert_end,
                                                         sorted, wgt, top, I, K, act, limit);
+  else
+    return PTL_ERR_ARG;
+  return ptl_launch_status();
+}
+
+// out [A, I] (sorted order) = act(w_a * x[token] Wu_e^T) for experts without a gate; w [E, I, K];
+// wgt null: the routing weight is not applied here.
+extern "C" int ptl_moe_up(void* out, long ldo, const void* x, long ldx, const void* w,
+                          const int32_t* tile_expert, const int32_t* tile_row0, const int32_t* expert_end,
+                          const int32_t* sorted, const float* wgt, int max_tiles, int pairs, int top, int I,
+                          int K, int act, int dtype, hipStream_t st) {
+  if (max_tiles <= 0) return PTL_OK;
+  if (I <= 0 || K <= 0 || top <= 0 || max_tiles > 65535 || act != 2) return PTL_ERR_ARG;
+  dim3 grid((I + 63) / 64, max_tiles);
+  if (dtype == PTL_DTYPE_F32)
+    moe_gemm_kernel<float, MODE_UP><<<grid, 256, 0, st>>>((float*)out, ldo, (const float*)x, ldx,
+                                                          (const float*)w, tile_expert, tile_row0, expert_end,
+                                                          sorted, wgt, top, I, K, act, 0.f);
+  else if (dtype == PTL_DTYPE_BF16 && mfma_ok(x, ldx, w, K) && pairs >= MOE_TILED_FROM && K % TB_K == 0) {
+    dim3 wide((I + TB_BROWS - 1) / TB_BROWS, max_tiles);
+    moe_gemm_tiled_kernel<MODE_UP><<<wide, 256, 0, st>>>((bf16_t*)out, ldo, (const bf16_t*)x, ldx,
+                                                         (const bf16_t*)w, tile_expert, tile_row0, expert_end,
+                                                         sorted, wgt, top, I, K, act, 0.f);
+  } else if (dtype == PTL_DTYPE_BF16 && mfma_ok(x, ldx, w, K))
+    moe_gemm_mfma_kernel<MODE_UP><<<grid, 256, 0, st>>>((bf16_t*)out, ldo, (const bf16_t*)x, ldx,
+                                                        (const bf16_t*)w, tile_expert, tile_row0, expert_end,
+                                                        sorted, wgt, top, I, K, act, 0.f);
+  else if (dtype == PTL_DTYPE_BF16)
+    moe_gemm_kernel<bf16_t, MODE_UP><<<grid, 256, 0, st>>>((bf16_t*)out, ldo, (const bf16_t*)x, ldx,
+                                                           (const bf16_t*)w, tile_expert, tile_row0,
+                                                           expert_end, sorted, wgt, top, I, K, act, 0.f);
   else
     return PTL_ERR_ARG;
   return ptl_launch_status();
@@ -550,20 +663,20 @@ extern "C" int ptl_moe_down(void* out, long ldo, const void* x, long ldx, const 
   if (N <= 0 || K <= 0 || max_tiles > 65535) return PTL_ERR_ARG;
   dim3 grid((N + 63) / 64, max_tiles);
   if (dtype == PTL_DTYPE_F32)
-    moe_gemm_kernel<float, false><<<grid, 256, 0, st>>>((float*)out, ldo, (const float*)x, ldx, (const float*)w,
+    moe_gemm_kernel<float, MODE_DOWN><<<grid, 256, 0, st>>>((float*)out, ldo, (const float*)x, ldx, (const float*)w,
                                                         tile_expert, tile_row0, expert_end, nullptr, nullptr, 1,
                                                         N, K, 0, 0.f);
   else if (dtype == PTL_DTYPE_BF16 && mfma_ok(x, ldx, w, K) && pairs >= MOE_TILED_FROM && K % TB_K == 0) {
     dim3 wide((N + TB_BROWS - 1) / TB_BROWS, max_tiles);
-    moe_gemm_tiled_kernel<false><<<wide, 256, 0, st>>>((bf16_t*)out, ldo, (const bf16_t*)x, ldx,
+    moe_gemm_tiled_kernel<MODE_DOWN><<<wide, 256, 0, st>>>((bf16_t*)out, ldo, (const bf16_t*)x, ldx,
                                                        (const bf16_t*)w, tile_expert, tile_row0, expert_end,
                                                        nullptr, nullptr, 1, N, K, 0, 0.f);
   } else if (dtype == PTL_DTYPE_BF16 && mfma_ok(x, ldx, w, K))
-    moe_gemm_mfma_kernel<false><<<grid, 256, 0, st>>>((bf16_t*)out, ldo, (const bf16_t*)x, ldx,
+    moe_gemm_mfma_kernel<MODE_DOWN><<<grid, 256, 0, st>>>((bf16_t*)out, ldo, (const bf16_t*)x, ldx,
                                                       (const bf16_t*)w, tile_expert, tile_row0, expert_end,
                                                       nullptr, nullptr, 1, N, K, 0, 0.f);
   else if (dtype == PTL_DTYPE_BF16)
-    moe_gemm_kernel<bf16_t, false><<<grid, 256, 0, st>>>((bf16_t*)out, ldo, (const bf16_t*)x, ldx,
+    moe_gemm_kernel<bf16_t, MODE_DOWN><<<grid, 256, 0, st>>>((bf16_t*)out, ldo, (const bf16_t*)x, ldx,
                                                          (const bf16_t*)w, tile_expert, tile_row0, expert_end,
                                                          nullptr, nullptr, 1, N, K, 0, 0.f);
   else
@@ -571,25 +684,31 @@ extern "C" int ptl_moe_down(void* out, long ldo, const void* x, long ldx, const 
   return ptl_launch_status();
 }
 
-// y[t, :] = sum_k f_k * rows[pos_of[t * top + k], :] + gate[t * ldg] * shared[t, :], float32.
-// f_k = wgt[t * top + k] when wgt is given (the weight scales the expert's output), else 1.
+// y[t, :] = sum_k f_k * rows[pos_of[t * top + k], :] + gate[t * ldg] * shared[t, :]
+//           + ident[t] * xin[t, :], float32.
+// f_k = wgt[t * top + k] when wgt is given (the weight scales the expert's output), else 1. A pair
+// with pos_of < 0 has no row (its expert returns its input: that is the last term).
 template <typename T>
 __global__ void __launch_bounds__(256)
 moe_combine_kernel(float* __restrict__ y, const T* __restrict__ rows, long ldr, const int32_t* __restrict__ pos_of,
                    const float* __restrict__ wgt, int top, const T* __restrict__ shared,
-                   const float* __restrict__ gate, int ldg, int N) {
+                   const float* __restrict__ gate, int ldg, const T* __restrict__ xin, long ldx,
+                   const float* __restrict__ ident, int N) {
   const size_t t = blockIdx.y;
   const int n = blockIdx.x * 256 + threadIdx.x;
   if (n >= N) return;
   float s = 0.f;
   for (int k = 0; k < top; ++k) {
-    const float v = to_float<T>(rows[(size_t)pos_of[t * top + k] * ldr + n]);
+    const int p = pos_of[t * top + k];
+    if (p < 0) continue;
+    const float v = to_float<T>(rows[(size_t)p * ldr + n]);
     s += wgt ? v * wgt[t * top + k] : v;
   }
   if (shared) {
     const float v = to_float<T>(shared[t * N + n]);
     s += gate ? v * gate[t * ldg] : v;
   }
+  if (ident) s = fmaf(ident[t], to_float<T>(xin[t * ldx + n]), s);
   y[t * N + n] = s;
 }
 
@@ -597,7 +716,8 @@ moe_combine_kernel(float* __restrict__ y, const T* __restrict__ rows, long ldr, 
 __global__ void __launch_bounds__(256)
 moe_combine_bf16_vec_kernel(float* __restrict__ y, const bf16_t* __restrict__ rows, long ldr,
                             const int32_t* __restrict__ pos_of, const float* __restrict__ wgt, int top,
-                            const bf16_t* __restrict__ shared, const float* __restrict__ gate, int ldg, int N8) {
+                            const bf16_t* __restrict__ shared, const float* __restrict__ gate, int ldg,
+                            const bf16_t* __restrict__ xin, long ldx, const float* __restrict__ ident, int N8) {
   const size_t t = blockIdx.y;
   const int c = blockIdx.x * 256 + threadIdx.x;
   if (c >= N8) return;
@@ -606,8 +726,10 @@ moe_combine_bf16_vec_kernel(float* __restrict__ y, const bf16_t* __restrict__ ro
   for (int j = 0; j < 8; ++j) s[j] = 0.f;
   union V { uint4 u; bf16_t e[8]; };
   for (int k = 0; k < top; ++k) {
+    const int p = pos_of[t * top + k];
+    if (p < 0) continue;
     V v;
-    v.u = load_once(rows + (size_t)pos_of[t * top + k] * ldr + 8 * c);
+    v.u = load_once(rows + (size_t)p * ldr + 8 * c);
     const float f = wgt ? wgt[t * top + k] : 1.f;
 #pragma unroll
     for (int j = 0; j < 8; ++j) s[j] += bf16_to_float(v.e[j]) * f;
@@ -619,36 +741,48 @@ moe_combine_bf16_vec_kernel(float* __restrict__ y, const bf16_t* __restrict__ ro
 #pragma unroll
     for (int j = 0; j < 8; ++j) s[j] += bf16_to_float(v.e[j]) * f;
   }
+  if (ident) {
+    V v;
+    v.u = *reinterpret_cast<const uint4*>(xin + t * ldx + 8 * c);
+    const float f = ident[t];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) s[j] = fmaf(f, bf16_to_float(v.e[j]), s[j]);
+  }
   float4* dst = reinterpret_cast<float4*>(y + (t * N8 + c) * 8);
   dst[0] = make_float4(s[0], s[1], s[2], s[3]);
   dst[1] = make_float4(s[4], s[5], s[6], s[7]);
 }
 
+// ident [T] with xin [T, N] (row stride ldx, the rows' dtype) or both null
 extern "C" int ptl_moe_combine(float* y, const void* rows, long ldr, const int32_t* pos_of, const float* wgt,
-                               int top, const void* shared, const float* gate, int ldg, int T_, int N, int dtype,
-                               hipStream_t st) {
+                               int top, const void* shared, const float* gate, int ldg, const void* xin,
+                               long ldx, const float* ident, int T_, int N, int dtype, hipStream_t st) {
   if (T_ <= 0) return PTL_OK;
-  if (N <= 0 || top <= 0 || T_ > 65535 * 64) return PTL_ERR_ARG;
+  if (N <= 0 || top <= 0 || T_ > 65535 * 64 || (ident && !xin)) return PTL_ERR_ARG;
   for (int t0 = 0; t0 < T_; t0 += 65535) {
     const int nt = T_ - t0 < 65535 ? T_ - t0 : 65535;
     dim3 grid((N + 255) / 256, nt);
     const size_t o = (size_t)t0;
-    if (dtype == PTL_DTYPE_BF16 && N % 8 == 0 && ldr % 8 == 0 &&
-        ((uintptr_t)rows | (uintptr_t)shared) % 16 == 0 && (uintptr_t)y % 16 == 0) {
+    if (dtype == PTL_DTYPE_BF16 && N % 8 == 0 && ldr % 8 == 0 && (!ident || ldx % 8 == 0) &&
+        ((uintptr_t)rows | (uintptr_t)shared | (uintptr_t)(ident ? xin : nullptr)) % 16 == 0 &&
+        (uintptr_t)y % 16 == 0) {
       dim3 vgrid((N / 8 + 255) / 256, nt);
       moe_combine_bf16_vec_kernel<<<vgrid, 256, 0, st>>>(
           y + o * N, (const bf16_t*)rows, ldr, pos_of + o * top, wgt ? wgt + o * top : nullptr, top,
-          shared ? (const bf16_t*)shared + o * N : nullptr, gate ? gate + o * ldg : nullptr, ldg, N / 8);
+          shared ? (const bf16_t*)shared + o * N : nullptr, gate ? gate + o * ldg : nullptr, ldg,
+          ident ? (const bf16_t*)xin + o * ldx : nullptr, ldx, ident ? ident + o : nullptr, N / 8);
       continue;
     }
     if (dtype == PTL_DTYPE_F32)
       moe_combine_kernel<float><<<grid, 256, 0, st>>>(
           y + o * N, (const float*)rows, ldr, pos_of + o * top, wgt ? wgt + o * top : nullptr, top,
-          shared ? (const float*)shared + o * N : nullptr, gate ? gate + o * ldg : nullptr, ldg, N);
+          shared ? (const float*)shared + o * N : nullptr, gate ? gate + o * ldg : nullptr, ldg,
+          ident ? (const float*)xin + o * ldx : nullptr, ldx, ident ? ident + o : nullptr, N);
     else if (dtype == PTL_DTYPE_BF16)
       moe_combine_kernel<bf16_t><<<grid, 256, 0, st>>>(
           y + o * N, (const bf16_t*)rows, ldr, pos_of + o * top, wgt ? wgt + o * top : nullptr, top,
-          shared ? (const bf16_t*)shared + o * N : nullptr, gate ? gate + o * ldg : nullptr, ldg, N);
+          shared ? (const bf16_t*)shared + o * N : nullptr, gate ? gate + o * ldg : nullptr, ldg,
+          ident ? (const bf16_t*)xin + o * ldx : nullptr, ldx, ident ? ident + o : nullptr, N);
     else
       return PTL_ERR_ARG;
   }
@@ -700,6 +834,50 @@ extern "C" int ptl_gated_act(void* out, const void* gate_up, int T_, int I, int 
     gated_act_kernel<float><<<(int)blocks, 256, 0, st>>>((float*)out, (const float*)gate_up, I, total, act, limit);
   else if (dtype == PTL_DTYPE_BF16)
     gated_act_kernel<bf16_t><<<(int)blocks, 256, 0, st>>>((bf16_t*)out, (const bf16_t*)gate_up, I, total, act, limit);
+  else
+    return PTL_ERR_ARG;
+  return ptl_launch_status();
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+unary_act_kernel(T* __restrict__ out, const T* __restrict__ in, size_t total, int act) {
+  size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  const size_t step = (size_t)gridDim.x * 256;
+  for (; i < total; i += step) out[i] = from_float<T>(unary_act(act, to_float<T>(in[i])));
+}
+
+// bfloat16 with a total that is a multiple of 8: 16-byte loads (marked as read once) and stores
+__global__ void __launch_bounds__(256)
+unary_act_bf16_vec_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ in, size_t total8, int act) {
+  size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  const size_t step = (size_t)gridDim.x * 256;
+  for (; i < total8; i += step) {
+    union { uint4 u; bf16_t e[8]; } v, o;
+    v.u = load_once(in + i * 8);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) o.e[j] = float_to_bf16(unary_act(act, bf16_to_float(v.e[j])));
+    *reinterpret_cast<uint4*>(out + i * 8) = o.u;
+  }
+}
+
+// out [T, I] = act(in) for a dense up product of an expert without a gate (act 2: relu(u)^2)
+extern "C" int ptl_unary_act(void* out, const void* in, int T_, int I, int act, int dtype, hipStream_t st) {
+  if (T_ <= 0) return PTL_OK;
+  if (I <= 0 || act != 2) return PTL_ERR_ARG;
+  const size_t total = (size_t)T_ * I;
+  if (dtype == PTL_DTYPE_BF16 && total % 8 == 0 && ((uintptr_t)out | (uintptr_t)in) % 16 == 0) {
+    size_t blocks = (total / 8 + 255) / 256;
+    if (blocks > 65536) blocks = 65536;
+    unary_act_bf16_vec_kernel<<<(int)blocks, 256, 0, st>>>((bf16_t*)out, (const bf16_t*)in, total / 8, act);
+    return ptl_launch_status();
+  }
+  size_t blocks = (total + 255) / 256;
+  if (blocks > 65536) blocks = 65536;
+  if (dtype == PTL_DTYPE_F32)
+    unary_act_kernel<float><<<(int)blocks, 256, 0, st>>>((float*)out, (const float*)in, total, act);
+  else if (dtype == PTL_DTYPE_BF16)
+    unary_act_kernel<bf16_t><<<(int)blocks, 256, 0, st>>>((bf16_t*)out, (const bf16_t*)in, total, act);
   else
     return PTL_ERR_ARG;
   return ptl_launch_status();

@@ -12,7 +12,10 @@
 // ptl_stream_add_rmsnorm_sum: the same for a result that is a weighted sum of two and a bias.
 // ptl_stream_rmsnorm: the RMS norm of rows of the stream, in the engine's type.
 // ptl_dyt: the norm alone, for rows that are no stream (the rows picked for the head).
-// ptl_embedding_scaled: stream[t] = table[ids[t]] * scale, in float32.
+// ptl_embedding_scaled: stream[t] = table[ids[t]] * scale, in float32 (``copies`` times side by side in
+//   a row, for a model that keeps several streams).
+// ptl_hyper_mix: several residual streams a token (hyper-connections): the streams' update behind a
+//   sublayer and the read-out with its RMS norm in front of the next one (where it stands, below).
 // ptl_gelu_gather_mul: out[t, j] = gelu_tanh(z[t, j]) * table[ids[t], col0 + j]: a gate on a
 //   per-token vector looked up in a table that several layers share.
 //
@@ -227,24 +230,28 @@ extern "C" int ptl_stream_rmsnorm(void* out, int out_dtype, const float* x, cons
 
 template <typename T>
 __global__ void embedding_scaled_kernel(float* __restrict__ out, const T* __restrict__ table,
-                                        const int32_t* __restrict__ ids, int H, int V, float scale) {
+                                        const int32_t* __restrict__ ids, int H, int V, float scale,
+                                        int copies) {
   const int t = blockIdx.x;
   int id = ids[t];
   if (id < 0 || id >= V) id = 0;          // checked on the host; never read out of bounds
   const T* src = table + (size_t)id * H;
-  float* dst = out + (size_t)t * H;
-  for (int i = threadIdx.x; i < H; i += blockDim.x) dst[i] = to_float<T>(src[i]) * scale;
+  float* dst = out + (size_t)t * H * copies;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) {
+    const float v = to_float<T>(src[i]) * scale;
+    for (int s = 0; s < copies; ++s) dst[(size_t)s * H + i] = v;
+  }
 }
 
 extern "C" int ptl_embedding_scaled(float* out, const void* table, const int32_t* ids, int T_, int H,
-                                    int V, float scale, int dtype, hipStream_t st) {
+                                    int V, float scale, int copies, int dtype, hipStream_t st) {
   if (T_ <= 0) return PTL_OK;
-  if (H <= 0 || V <= 0) return PTL_ERR_ARG;
+  if (H <= 0 || V <= 0 || copies < 1) return PTL_ERR_ARG;
   const int threads = H >= 1024 ? 256 : (H >= 256 ? 128 : 64);
   if (dtype == PTL_DTYPE_F32)
-    embedding_scaled_kernel<float><<<T_, threads, 0, st>>>(out, (const float*)table, ids, H, V, scale);
+    embedding_scaled_kernel<float><<<T_, threads, 0, st>>>(out, (const float*)table, ids, H, V, scale, copies);
   else if (dtype == PTL_DTYPE_BF16)
-    embedding_scaled_kernel<bf16_t><<<T_, threads, 0, st>>>(out, (const bf16_t*)table, ids, H, V, scale);
+    embedding_scaled_kernel<bf16_t><<<T_, threads, 0, st>>>(out, (const bf16_t*)table, ids, H, V, scale, copies);
   else
     return PTL_ERR_ARG;
   return ptl_launch_status();
@@ -285,4 +292,108 @@ extern "C" int ptl_gelu_gather_mul(void* out, const void* z, const void* table, 
   else
     return PTL_ERR_ARG;
   return ptl_launch_status();
+}
+
+// Hyper-connections: a token has S residual streams x_1 .. x_S, [T, S, H] float32. Around a sublayer
+//
+//   u = sum_s in[s] x_s;   y = sublayer(rmsnorm(u) w);   x_t <- sum_s mix[s, t] x_s + out[t] y
+//
+// (all streams at once from the old ones). One kernel makes the update behind a sublayer and the
+// read-out in front of the next one: with y, the streams are updated in place; with nw, u is read
+// from the (new) streams and normed into ``out``. Either half may be absent. Null coefficients
+// stand for a single plain stream: in = ones, mix = the identity, out = ones (then S = 1 is the
+// residual sum in front of a norm, and in = ones alone is the sum of the streams). One workgroup
+// a token; u waits in LDS between the pass that makes it and the one that scales it.
+#define HYPER_MAX_S 16
+
+template <int SM, typename TY, typename TO>
+__global__ void __launch_bounds__(256)
+hyper_mix_kernel(float* __restrict__ streams, const TY* __restrict__ y, const float* __restrict__ mix,
+                 const float* __restrict__ outc, const float* __restrict__ inc, const float* __restrict__ nw,
+                 float eps, TO* __restrict__ out, int S, int H) {
+  extern __shared__ float us[];            // [H]
+  __shared__ float scratch[16];
+  __shared__ float cm[HYPER_MAX_S * HYPER_MAX_S], co[HYPER_MAX_S], ci[HYPER_MAX_S];
+  const int tid = threadIdx.x;
+  if (tid < S * S) cm[tid] = mix ? mix[tid] : (tid / S == tid % S ? 1.f : 0.f);
+  if (tid < S) {
+    co[tid] = outc ? outc[tid] : 1.f;
+    ci[tid] = inc ? inc[tid] : 1.f;
+  }
+  __syncthreads();
+  float* row = streams + (size_t)blockIdx.x * S * H;
+  float ss = 0.f;
+  for (int c = tid; c < H; c += 256) {
+    float x[SM];
+#pragma unroll
+    for (int s = 0; s < SM; ++s) x[s] = s < S ? row[(size_t)s * H + c] : 0.f;
+    if (y) {
+      const float v = to_float<TY>(y[(size_t)blockIdx.x * H + c]);
+      float nx[SM];
+#pragma unroll
+      for (int t = 0; t < SM; ++t) {
+        float a = co[t] * v;
+#pragma unroll
+        for (int s = 0; s < SM; ++s) a = fmaf(s < S && t < S ? cm[s * S + t] : 0.f, x[s], a);
+        nx[t] = a;
+      }
+#pragma unroll
+      for (int t = 0; t < SM; ++t) {
+        x[t] = nx[t];
+        if (t < S) row[(size_t)t * H + c] = nx[t];
+      }
+    }
+    if (nw) {
+      float u = 0.f;
+#pragma unroll
+      for (int s = 0; s < SM; ++s) u = fmaf(s < S ? ci[s] : 0.f, x[s], u);
+      us[c] = u;
+      ss = fmaf(u, u, ss);
+    }
+  }
+  if (!nw) return;
+  ss = block_sum(ss, scratch);
+  const float r = 1.0f / sqrtf(ss / (float)H + eps);
+  for (int c = tid; c < H; c += 256) out[(size_t)blockIdx.x * H + c] = from_float<TO>(us[c] * r * nw[c]);
+}
+
+template <typename TY, typename TO>
+static int launch_hyper(float* streams, const void* y, const float* mix, const float* outc, const float* inc,
+                        const float* nw, float eps, void* out, int T_, int S, int H, hipStream_t st) {
+  const size_t lds = nw ? (size_t)H * sizeof(float) : 0;
+#define GO(SM)                                                                                       \
+  {                                                                                                  \
+    if (lds > 48 * 1024 &&                                                                           \
+        hipFuncSetAttribute((const void*)hyper_mix_kernel<SM, TY, TO>,                               \
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)     \
+      return PTL_ERR_LAUNCH;                                                                         \
+    hyper_mix_kernel<SM, TY, TO><<<T_, 256, lds, st>>>(streams, (const TY*)y, mix, outc, inc, nw, eps, \
+                                                       (TO*)out, S, H);                              \
+    return ptl_launch_status();                                                                      \
+  }
+  if (S <= 1) GO(1)
+  if (S <= 2) GO(2)
+  if (S <= 4) GO(4)
+  if (S <= 8) GO(8)
+  GO(16)
+#undef GO
+}
+
+// streams [T, S, H] float32 (updated in place when y is given); y [T, H] of y_dtype or null; mix
+// [S, S] (from, to), outc [S], inc [S] float32 or null; nw [H] float32 or null: no read-out; out
+// [T, H] of out_dtype.
+extern "C" int ptl_hyper_mix(float* streams, const void* y, int y_dtype, const float* mix, const float* outc,
+                             const float* inc, const float* nw, float eps, void* out, int out_dtype, int T_,
+                             int S, int H, hipStream_t st) {
+  if (T_ <= 0) return PTL_OK;
+  if (H <= 0 || S < 1 || S > HYPER_MAX_S || !streams || (nw && !out) || (!y && !nw) ||
+      (size_t)H * sizeof(float) > 150 * 1024)
+    return PTL_ERR_ARG;
+#define GO(TY, TO) return launch_hyper<TY, TO>(streams, y, mix, outc, inc, nw, eps, out, T_, S, H, st)
+  if (y_dtype == PTL_DTYPE_F32 && out_dtype == PTL_DTYPE_F32) GO(float, float);
+  if (y_dtype == PTL_DTYPE_F32 && out_dtype == PTL_DTYPE_BF16) GO(float, bf16_t);
+  if (y_dtype == PTL_DTYPE_BF16 && out_dtype == PTL_DTYPE_BF16) GO(bf16_t, bf16_t);
+  if (y_dtype == PTL_DTYPE_BF16 && out_dtype == PTL_DTYPE_F32) GO(bf16_t, float);
+#undef GO
+  return PTL_ERR_ARG;
 }

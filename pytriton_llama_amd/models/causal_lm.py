@@ -140,7 +140,10 @@ class CausalLM:
             # a block may leave its last product to the norm that comes next, if that norm can
             # take it (parts/base.py); the rows for the final norm are picked first, so not there
             after = self.blocks[self.schedule[i + 1].block] if i < last else None
-            if (after is not None and getattr(block, "can_defer_output", False)
+            if getattr(block, "takes_next_block", False):
+                # a block whose last kernel also does the first work of the block that runs next
+                h, residual = block.forward(h, residual, ctx, cache, next_block=after)
+            elif (after is not None and getattr(block, "can_defer_output", False)
                     and getattr(after, "takes_pending_product", False)):
                 h, residual = block.forward(h, residual, ctx, cache, defer_output=True)
             else:

@@ -940,18 +940,56 @@ def _check_stream(stream: torch.Tensor, what: str):
     return stream.shape
 
 
-def embedding_scaled(table: torch.Tensor, ids: torch.Tensor, scale: float) -> torch.Tensor:
-    """out[t] = table[ids[t]] * scale as float32 (the start of a float32 residual stream)."""
+def embedding_scaled(table: torch.Tensor, ids: torch.Tensor, scale: float, copies: int = 1) -> torch.Tensor:
+    """out[t] = table[ids[t]] * scale as float32 (the start of a float32 residual stream),
+    ``copies`` times side by side in a row (a model that keeps several streams a token)."""
     _need_gpu(table, ids)
     _i32(ids, "ids")
     if table.dim() != 2 or not table.is_contiguous():
         raise KernelError("embedding table must be a contiguous [V, H] matrix")
     V, H = table.shape
     T = ids.numel()
-    out = torch.empty((T, H), dtype=torch.float32, device=table.device)
+    if copies < 1:
+        raise KernelError("embedding_scaled: at least one copy")
+    out = torch.empty((T, copies * H), dtype=torch.float32, device=table.device)
     _check(library.load("stream").ptl_embedding_scaled(_ptr(out), _ptr(table), _ptr(ids), T, H, V,
-                                                       ctypes.c_float(scale), _dtype_code(table), _stream()),
-           "embedding_scaled")
+                                                       ctypes.c_float(scale), int(copies), _dtype_code(table),
+                                                       _stream()), "embedding_scaled")
+    return out
+
+
+HYPER_MAX_STREAMS = 16
+
+
+def hyper_mix(streams: torch.Tensor, num_streams: int, y: Optional[torch.Tensor] = None, mix=None, outc=None,
+              inc=None, norm_weight: Optional[torch.Tensor] = None, eps: float = 0.0,
+              out_dtype: Optional[torch.dtype] = None) -> Optional[torch.Tensor]:
+    """Several residual streams a token, ``streams`` float32 [T, S * H] (stream after stream in a
+    row). With ``y`` [T, H]: x_t <- sum_s mix[s, t] x_s + outc[t] y for all t at once, in place. With
+    ``norm_weight`` [H]: returns rmsnorm(sum_s inc[s] x_s) * norm_weight in ``out_dtype``, read from
+    the streams as the update left them. Coefficients are float32 device tensors; None stands for
+    the identity (mix), ones (outc, inc)."""
+    S = int(num_streams)
+    T, SH = _check_stream(streams, "hyper_mix")
+    if not 1 <= S <= HYPER_MAX_STREAMS or SH % S:
+        raise KernelError(f"hyper_mix: {S} streams do not divide a row of {SH} (at most {HYPER_MAX_STREAMS})")
+    H = SH // S
+    if y is None and norm_weight is None:
+        raise KernelError("hyper_mix: nothing to do")
+    if y is not None:
+        _need_gpu(y)
+        if y.shape != (T, H) or not y.is_contiguous():
+            raise KernelError(f"hyper_mix: y must be a contiguous [{T}, {H}] matrix")
+    for c, n, what in ((mix, S * S, "mix"), (outc, S, "outc"), (inc, S, "inc"), (norm_weight, H, "norm_weight")):
+        if c is not None:
+            _f32_vec(c, n, f"hyper_mix: {what}")
+    out = None
+    if norm_weight is not None:
+        out = torch.empty((T, H), dtype=out_dtype or torch.float32, device=streams.device)
+    _check(library.load("stream").ptl_hyper_mix(
+        _ptr(streams), _ptr(y), _dtype_code(y) if y is not None else _F32, _ptr(mix), _ptr(outc), _ptr(inc),
+        _ptr(norm_weight), ctypes.c_float(eps), _ptr(out), _dtype_code(out) if out is not None else _F32,
+        T, S, H, _stream()), "hyper_mix")
     return out
 
 
@@ -1543,7 +1581,9 @@ def memory_scan(p: torch.Tensor, q_off: int, k_off: int, v_off: int, i_off: int,
 
 # ---------------------------------------------------------------------------
 # Routed experts (csrc/moe.hip)
-ACT_SILU, ACT_CLAMPED = 0, 1
+ACT_SILU, ACT_CLAMPED = 0, 1           # gated: act(gate) * up
+ACT_RELU2 = 2                          # no gate: relu(up)^2
+SCORE_SIGMOID, SCORE_SOFTMAX = 0, 1
 
 
 def gated_act(gate_up: torch.Tensor, act: int, limit: float = 0.0) -> torch.Tensor:
@@ -1561,19 +1601,31 @@ def gated_act(gate_up: torch.Tensor, act: int, limit: float = 0.0) -> torch.Tens
 class Routing:
     """Where the (token, choice) pairs of a step went: see csrc/moe.hip."""
     __slots__ = ("idx", "wgt", "extra", "pos_of", "sorted", "expert_end", "tile_expert", "tile_row0",
-                 "max_tiles", "top", "experts")
+                 "max_tiles", "top", "experts", "ident")
 
 
 def moe_route(logits: torch.Tensor, experts: int, top: int, extra: int = 0,
-              renormalize: bool = False) -> Routing:
-    """Route every row of float32 ``logits`` [T, experts + extra] to its ``top`` experts by the
-    sigmoid of its logits and order the pairs by expert."""
+              renormalize: bool = False, score: int = SCORE_SIGMOID, correction: Optional[torch.Tensor] = None,
+              identity: int = 0, renorm_eps: float = 0.0, weight_scale: float = 1.0) -> Routing:
+    """Route every row of float32 ``logits`` [T, experts + identity + extra] to ``top`` of its
+    ``experts + identity`` router outputs and order the pairs by expert. Scores: the sigmoid of
+    the logits, or their softmax over the router outputs; the choice goes by score +
+    ``correction`` [experts + identity] when one is given; the weights are the scores
+    (``renormalize``: divided by their sum + renorm_eps) times weight_scale. The last
+    ``identity`` outputs are experts that return their input: their pairs take no part in the
+    products, and ``ident`` [T] holds the sum of their weights a token."""
     _need_gpu(logits)
     if logits.dim() != 2 or logits.dtype != torch.float32 or logits.stride(1) != 1 \
             or logits.shape[1] < experts + extra:
         raise KernelError("moe_route: logits must be float32 [T, experts + extra] with dense rows")
-    if not 0 < top <= experts or experts > 1024 or not 0 <= extra <= 64:
-        raise KernelError(f"moe_route: {top} of {experts} experts (+{extra}) is not a case the kernel takes")
+    outputs = experts + identity
+    if identity < 0 or logits.shape[1] < outputs + extra:
+        raise KernelError("moe_route: logits must be float32 [T, experts + identity + extra]")
+    if not 0 < top <= outputs or outputs > 1024 or not 0 <= extra <= 64 or experts < 1:
+        raise KernelError(f"moe_route: {top} of {experts} + {identity} experts (+{extra}) is not a case the "
+                          "kernel takes")
+    if correction is not None:
+        _f32_vec(correction, outputs, "moe_route: correction")
     T = logits.shape[0]
     A = T * top
     lib = library.load("moe")
@@ -1588,8 +1640,11 @@ def moe_route(logits: torch.Tensor, experts: int, top: int, extra: int = 0,
     r.tile_row0 = ints[3 * A + experts + r.max_tiles:]
     r.wgt = torch.empty(A, dtype=torch.float32, device=dev)
     r.extra = torch.empty((T, extra), dtype=torch.float32, device=dev) if extra else None
-    _check(lib.ptl_moe_topk(_ptr(logits), int(logits.stride(0)), T, experts, top, extra, int(renormalize),
-                            _ptr(r.idx), _ptr(r.wgt), _ptr(r.extra), _stream()), "moe_topk")
+    r.ident = torch.empty(T, dtype=torch.float32, device=dev) if identity else None
+    _check(lib.ptl_moe_topk(_ptr(logits), int(logits.stride(0)), T, outputs, top, extra, int(renormalize),
+                            int(score), _ptr(correction), experts, ctypes.c_float(renorm_eps),
+                            ctypes.c_float(weight_scale), _ptr(r.idx), _ptr(r.wgt), _ptr(r.extra),
+                            _ptr(r.ident), _stream()), "moe_topk")
     _check(lib.ptl_moe_sort(_ptr(r.idx), A, experts, _ptr(r.pos_of), _ptr(r.sorted), _ptr(r.expert_end),
                             _ptr(r.tile_expert), _ptr(r.tile_row0), r.max_tiles, _stream()), "moe_sort")
     return r
@@ -1598,13 +1653,19 @@ def moe_route(logits: torch.Tensor, experts: int, top: int, extra: int = 0,
 def moe_experts(x: torch.Tensor, r: Routing, gate_up: torch.Tensor, down: torch.Tensor, act: int,
                 limit: float, weight_on_input: bool, shared: Optional[torch.Tensor] = None,
                 shared_gate: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """The routed experts on x [T, K]: gate_up [E, 2 I, K], down [E, N, I]; returns float32
-    [T, N] = sum over a row's choices of its experts' outputs (+ shared_gate[t] * shared[t])."""
+    """The routed experts on x [T, K]: gate_up [E, 2 I, K] (for an activation without a gate,
+    ACT_RELU2: the up matrices [E, I, K]), down [E, N, I]; returns float32 [T, N] = sum over a
+    row's choices of its experts' outputs (+ shared_gate[t] * shared[t], + r.ident[t] * x[t] for
+    the experts that return their input)."""
     _need_gpu(x, gate_up, down, shared, shared_gate)
     T, K = x.shape
     E, I2, _ = gate_up.shape
-    I, N = I2 // 2, down.shape[1]
-    if x.stride(1) != 1 or gate_up.shape != (E, 2 * I, K) or down.shape != (E, N, I) or E != r.experts \
+    gated = act != ACT_RELU2
+    I, N = (I2 // 2 if gated else I2), down.shape[1]
+    if r.ident is not None and (N != K or weight_on_input):
+        raise KernelError("moe_experts: experts that return their input need a result of the input's size "
+                          "and weights on the output")
+    if x.stride(1) != 1 or gate_up.shape != (E, (2 if gated else 1) * I, K) or down.shape != (E, N, I) or E != r.experts \
             or not gate_up.is_contiguous() or not down.is_contiguous() \
             or not (x.dtype == gate_up.dtype == down.dtype) or r.idx.numel() != T * r.top:
         raise KernelError("moe_experts: shapes or dtypes do not fit the routing")
@@ -1617,10 +1678,16 @@ def moe_experts(x: torch.Tensor, r: Routing, gate_up: torch.Tensor, down: torch.
     A = T * r.top
     code = _dtype_code(x)
     mid = torch.empty((A, I), dtype=x.dtype, device=x.device)
-    _check(lib.ptl_moe_gate_up(_ptr(mid), ctypes.c_long(I), _ptr(x), ctypes.c_long(x.stride(0)), _ptr(gate_up),
-                               _ptr(r.tile_expert), _ptr(r.tile_row0), _ptr(r.expert_end), _ptr(r.sorted),
-                               _ptr(r.wgt) if weight_on_input else None, r.max_tiles, A, r.top, I, K, int(act),
-                               ctypes.c_float(limit), code, _stream()), "moe_gate_up")
+    if gated:
+        _check(lib.ptl_moe_gate_up(_ptr(mid), ctypes.c_long(I), _ptr(x), ctypes.c_long(x.stride(0)), _ptr(gate_up),
+                                   _ptr(r.tile_expert), _ptr(r.tile_row0), _ptr(r.expert_end), _ptr(r.sorted),
+                                   _ptr(r.wgt) if weight_on_input else None, r.max_tiles, A, r.top, I, K, int(act),
+                                   ctypes.c_float(limit), code, _stream()), "moe_gate_up")
+    else:
+        _check(lib.ptl_moe_up(_ptr(mid), ctypes.c_long(I), _ptr(x), ctypes.c_long(x.stride(0)), _ptr(gate_up),
+                              _ptr(r.tile_expert), _ptr(r.tile_row0), _ptr(r.expert_end), _ptr(r.sorted),
+                              _ptr(r.wgt) if weight_on_input else None, r.max_tiles, A, r.top, I, K, int(act),
+                              code, _stream()), "moe_up")
     rows = torch.empty((A, N), dtype=x.dtype, device=x.device)
     _check(lib.ptl_moe_down(_ptr(rows), ctypes.c_long(N), _ptr(mid), ctypes.c_long(I), _ptr(down),
                             _ptr(r.tile_expert), _ptr(r.tile_row0), _ptr(r.expert_end), r.max_tiles, A, N, I,
@@ -1628,6 +1695,106 @@ def moe_experts(x: torch.Tensor, r: Routing, gate_up: torch.Tensor, down: torch.
     y = torch.empty((T, N), dtype=torch.float32, device=x.device)
     _check(lib.ptl_moe_combine(_ptr(y), _ptr(rows), ctypes.c_long(N), _ptr(r.pos_of),
                                None if weight_on_input else _ptr(r.wgt), r.top, _ptr(shared), _ptr(shared_gate),
-                               int(shared_gate.stride(0)) if shared_gate is not None else 0, T, N, code,
-                               _stream()), "moe_combine")
+                               int(shared_gate.stride(0)) if shared_gate is not None else 0,
+                               _ptr(x) if r.ident is not None else None, ctypes.c_long(x.stride(0)),
+                               _ptr(r.ident), T, N, code, _stream()), "moe_combine")
     return y
+
+
+def unary_act(u: torch.Tensor, act: int = ACT_RELU2) -> torch.Tensor:
+    """An activation without a gate on a dense product [T, I] (ACT_RELU2: relu(u)^2)."""
+    _need_gpu(u)
+    if u.dim() != 2 or not u.is_contiguous():
+        raise KernelError("unary_act: input must be a contiguous [T, I] matrix")
+    out = torch.empty_like(u)
+    _check(library.load("moe").ptl_unary_act(_ptr(out), _ptr(u), u.shape[0], u.shape[1], int(act),
+                                             _dtype_code(u), _stream()), "unary_act")
+    return out
+
+
+# ---------------------------------------------------------------------------
+# The selective scan (csrc/selective.hip)
+def selective_state_floats(channels: int, state: int, taps: int) -> int:
+    """Floats of a state slot: the states [channels, state], then the convolution's last
+    taps - 1 inputs [taps - 1, channels]."""
+    return channels * state + (taps - 1) * channels
+
+
+def selective_conv(p: torch.Tensor, x_off: int, conv_weight: torch.Tensor, conv_bias: Optional[torch.Tensor],
+                   state: torch.Tensor, tail_off: int, q_start: torch.Tensor, state_slots: torch.Tensor,
+                   max_q_len: int, lp_dtype: Optional[torch.dtype] = None):
+    """silu(causal convolution over time + bias) of the channels p[:, x_off : x_off + C] (float32);
+    conv_weight float32 [C, taps], the last column is the current token's; inputs before the step's
+    first token come from the slots' tails [taps - 1, C] at tail_off. Returns (float32 [T, C], the
+    same in ``lp_dtype`` or None)."""
+    _f32_rows(p, "selective_conv: p")
+    _need_gpu(conv_weight, state, q_start, state_slots)
+    T = p.shape[0]
+    if conv_weight.dim() != 2:
+        raise KernelError("selective_conv: conv_weight must be [C, taps]")
+    C, taps = conv_weight.shape
+    _f32_vec(conv_weight, C * taps, "selective_conv: conv_weight")
+    if conv_bias is not None:
+        _f32_vec(conv_bias, C, "selective_conv: conv_bias")
+    if state.dim() != 2 or state.dtype != torch.float32 or not state.is_contiguous() or x_off < 0 \
+            or x_off + C > p.shape[1] or tail_off < 0 or tail_off + (taps - 1) * C > state.shape[1]:
+        raise KernelError("selective_conv: columns outside p, or the tail outside the state")
+    _i32(q_start, "q_start")
+    _i32(state_slots, "state_slots")
+    n = state_slots.numel()
+    if q_start.numel() != n + 1:
+        raise KernelError("selective_conv: q_start has one entry more than there are sequences")
+    xc = torch.empty((T, C), dtype=torch.float32, device=p.device)
+    lp = None
+    if lp_dtype is not None and lp_dtype != torch.float32:
+        lp = torch.empty((T, C), dtype=lp_dtype, device=p.device)
+    _check(library.load("selective").ptl_selective_conv(
+        _ptr(xc), _ptr(lp), _dtype_code(lp) if lp is not None else _F32, _ptr(p), ctypes.c_long(p.stride(0)),
+        int(x_off), _ptr(conv_weight), _ptr(conv_bias), int(taps), _ptr(state), ctypes.c_long(state.stride(0)),
+        ctypes.c_long(tail_off), _ptr(q_start), _ptr(state_slots), n, int(max_q_len), C, _stream()),
+        "selective_conv")
+    return xc, lp
+
+
+def selective_scan(xc: torch.Tensor, p: torch.Tensor, z_off: int, r: torch.Tensor, rank: int, b_off: int,
+                   c_off: int, w_dt: torch.Tensor, dt_bias: torch.Tensor, A_log: torch.Tensor, D: torch.Tensor,
+                   state: torch.Tensor, q_start: torch.Tensor, state_slots: torch.Tensor,
+                   out_dtype: torch.dtype) -> torch.Tensor:
+    """The recurrence S <- exp(dt A) S + dt x B, y = S C + D x, and the gate y * silu(z), for every
+    sequence of the step from its slot's state [C, N] (at the start of the slot), which it leaves
+    advanced. xc float32 [T, C]; z = p[:, z_off : z_off + C] (float32); r float32 rows with the
+    step input in columns 0..rank-1, B [N] at b_off, C [N] at c_off; w_dt [C, rank], dt_bias [C],
+    A_log [C, N], D [C] float32. Returns [T, C] in ``out_dtype``."""
+    _f32_rows(p, "selective_scan: p")
+    _f32_rows(r, "selective_scan: r")
+    _need_gpu(xc, w_dt, dt_bias, A_log, D, state, q_start, state_slots)
+    if xc.dim() != 2 or xc.dtype != torch.float32 or not xc.is_contiguous():
+        raise KernelError("selective_scan: xc must be a contiguous float32 [T, C] matrix")
+    T, C = xc.shape
+    if A_log.dim() != 2 or A_log.shape[0] != C:
+        raise KernelError(f"selective_scan: A_log must be [{C}, N]")
+    N, R = A_log.shape[1], int(rank)
+    _f32_vec(A_log, C * N, "selective_scan: A_log")
+    _f32_vec(w_dt, C * R, "selective_scan: w_dt")
+    _f32_vec(dt_bias, C, "selective_scan: dt_bias")
+    _f32_vec(D, C, "selective_scan: D")
+    if p.shape[0] != T or r.shape[0] != T or z_off < 0 or z_off + C > p.shape[1] or R < 1 or R > r.shape[1] \
+            or min(b_off, c_off) < 0 or max(b_off, c_off) + N > r.shape[1]:
+        raise KernelError("selective_scan: columns outside p or r")
+    if N > 256 or 4 * (16 * (R + 2 * N) + 16 * R + 1024) > 150 * 1024:
+        raise KernelError(f"selective_scan: {N} states and a step input of {R} are more than the kernel takes")
+    if state.dim() != 2 or state.dtype != torch.float32 or not state.is_contiguous() or state.shape[1] < C * N:
+        raise KernelError("selective_scan: the state slots must be contiguous float32 rows of at least C * N")
+    _i32(q_start, "q_start")
+    _i32(state_slots, "state_slots")
+    n = state_slots.numel()
+    if q_start.numel() != n + 1:
+        raise KernelError("selective_scan: q_start has one entry more than there are sequences")
+    out = torch.empty((T, C), dtype=out_dtype, device=xc.device)
+    z = p[:, z_off:]
+    _check(library.load("selective").ptl_selective_scan(
+        _ptr(out), _dtype_code(out), _ptr(xc), _ptr(z), ctypes.c_long(p.stride(0)), _ptr(r),
+        ctypes.c_long(r.stride(0)), int(b_off), int(c_off), _ptr(w_dt), _ptr(dt_bias), _ptr(A_log), _ptr(D),
+        _ptr(state), ctypes.c_long(state.stride(0)), _ptr(q_start), _ptr(state_slots), n, C, N, R, _stream()),
+        "selective_scan")
+    return out

@@ -4,7 +4,7 @@ from __future__ import annotations
 import torch
 
 from .. import ops
-from .base import Part, PendingSum, as_tensor, register_part, run_norm
+from .base import ParamSource, Part, PendingSum, as_tensor, place, register_part, run_norm
 
 
 @register_part("block", "prenorm")
@@ -266,3 +266,123 @@ class OutputNormBlock(Part):
         a = self._add(stream, y, self.norm1, dtype, True)
         y = self.feed_forward.forward(a)
         return stream, self._add(stream, y, self.norm2, dtype, not self.last)
+
+
+@register_part("block", "hyper_connections")
+class HyperConnectionBlock(Part):
+    """Pre-norm sublayers on several residual streams a token (hyper-connections; Zhu et al.,
+    "Hyper-Connections"): the block's ``h`` is float32 [T, streams * hidden], stream after stream
+    in a row. For the mixer and then the feed-forward (which is optional), with the sublayer's
+    coefficients ``in`` [streams], ``mix`` [streams, streams] (from, to) and ``out`` [streams]:
+
+        u = sum_s in[s] x_s;   y = sublayer(rmsnorm(u) w);   x_t <- sum_s mix[s, t] x_s + out[t] y
+
+    all streams at once from the old ones. ``learned`` False: no coefficients in the checkpoint;
+    one stream with in = mix = out = 1, which is x <- x + sublayer(rmsnorm(x) w) on a float32
+    stream. The update behind a sublayer and the read-out with the norm in front of the next one
+    are one kernel (ops.hyper_mix), also across blocks: the model tells the block which block runs
+    next (``next_block``), the block's last kernel reads and norms for that block's mixer, and the
+    result travels where other blocks carry a residual. Sublayers read the engine's dtype and may
+    return float32."""
+    takes_next_block = True
+
+    def __init__(self, hidden_size: int, streams: int, mixer: Part, mixer_norm: Part, feed_forward: Part = None,
+                 ffn_norm: Part = None, learned: bool = True, mixer_hc: str = "hc1.", ffn_hc: str = "hc2.",
+                 in_name: str = "in", mix_name: str = "mix", out_name: str = "out"):
+        if (feed_forward is None) != (ffn_norm is None):
+            raise ValueError("a feed-forward comes with its norm, or neither")
+        if not 1 <= streams <= ops.HYPER_MAX_STREAMS or (not learned and streams != 1):
+            raise ValueError(f"1 to {ops.HYPER_MAX_STREAMS} streams (one when no coefficients are learned), "
+                             f"got {streams}")
+        for n in (mixer_norm, ffn_norm):
+            if n is not None and not (hasattr(n, "weight") and hasattr(n, "eps")):
+                raise ValueError("the norms of this block are RMS norms (a weight and an eps)")
+        self.hidden_size, self.streams, self.learned = int(hidden_size), int(streams), bool(learned)
+        self.mixer, self.norm1 = mixer, mixer_norm
+        self.feed_forward, self.norm2 = feed_forward, ffn_norm
+        self.hc_prefixes = (mixer_hc, ffn_hc)
+        self.hc_names = (in_name, mix_name, out_name)
+        self.coef = [None, None]            # per sublayer (in, mix, out) on the device, or None
+        libs = ("stream",)
+        for p in self._parts():
+            libs += tuple(p.kernel_libraries)
+        self.kernel_libraries = tuple(dict.fromkeys(libs))
+
+    def children(self):
+        roles = {"mixer": self.mixer, "norm1": self.norm1, "feed_forward": self.feed_forward,
+                 "norm2": self.norm2, "connections": self if self.learned else None}
+        return {k: p for k, p in roles.items() if p is not None}
+
+    def _parts(self):
+        return [p for p in (self.mixer, self.norm1, self.feed_forward, self.norm2) if p is not None]
+
+    def cache_spec(self):
+        return self.mixer.cache_spec() if hasattr(self.mixer, "cache_spec") else None
+
+    def work_lists(self):
+        lists = ()
+        for p in self._parts():
+            if hasattr(p, "work_lists"):
+                lists += tuple(p.work_lists())
+        return tuple(dict.fromkeys(lists))
+
+    def make_decode_copies(self) -> int:
+        return sum(p.make_decode_copies() for p in self._parts() if hasattr(p, "make_decode_copies"))
+
+    @property
+    def graph_capturable(self) -> bool:
+        return all(getattr(p, "graph_capturable", True) for p in self._parts())
+
+    # the block's own tensors: the coefficients of its sublayers
+    def param_sources(self):
+        if not self.learned:
+            return []
+        S = self.streams
+        i, m, o = self.hc_names
+        out = []
+        for q, prefix in enumerate(self.hc_prefixes):
+            if q == 1 and self.feed_forward is None:
+                continue
+            out += [ParamSource(prefix + i, (S,), "vector", init=("normal", 1.0 / S, 0.1)),
+                    ParamSource(prefix + o, (S,), "vector", init=("normal", 1.0, 0.1)),
+                    ParamSource(prefix + m, (S, S), "vector", init=("normal", 1.0 / S, 0.15))]
+        return out
+
+    def load(self, tensors, dtype, device) -> None:
+        if not self.learned:
+            return
+        i, m, o = self.hc_names
+        for q, prefix in enumerate(self.hc_prefixes):
+            if prefix + i in tensors:
+                self.coef[q] = tuple(place(tensors[prefix + n], "vector", dtype, device) for n in (i, m, o))
+
+    def read_args(self):
+        """(in coefficients or None, norm weight, eps) of the read-out in front of the mixer."""
+        c = self.coef[0]
+        return (c[0] if c is not None else None, self.norm1.weight, self.norm1.eps)
+
+    def _step(self, streams, y, q, nxt, dtype):
+        """The update behind sublayer ``q`` (y None: none) and the read-out ``nxt`` = (in, weight,
+        eps) in front of what follows (None: none)."""
+        c = self.coef[q] if y is not None else None
+        if isinstance(y, PendingSum) and len(y.terms) == 1 and y.terms[0][1] == 1.0 and y.bias is None:
+            y = y.terms[0][0]
+        if y is not None:
+            y = as_tensor(y)
+        inc, w, eps = nxt if nxt is not None else (None, None, 0.0)
+        return ops.hyper_mix(streams, self.streams, y, c[1] if c is not None else None,
+                             c[2] if c is not None else None, inc, w, eps, dtype)
+
+    def forward(self, h, residual, ctx, cache, next_block=None):
+        if h.dtype != torch.float32 or h.shape[1] != self.streams * self.hidden_size:
+            raise ops.KernelError(f"a hyper-connection block runs on float32 rows of {self.streams} streams")
+        streams, dtype = h, self.norm1.dtype
+        a = residual if residual is not None else self._step(streams, None, 0, self.read_args(), dtype)
+        y = self.mixer.forward(a, ctx, cache)
+        after = next_block.read_args() if isinstance(next_block, HyperConnectionBlock) else None
+        if self.feed_forward is None:
+            return streams, self._step(streams, y, 0, after, dtype)
+        c = self.coef[1]
+        a = self._step(streams, y, 0, (c[0] if c is not None else None, self.norm2.weight, self.norm2.eps), dtype)
+        y = self.feed_forward.forward(a)
+        return streams, self._step(streams, y, 1, after, dtype)

@@ -18,9 +18,13 @@ class TokenEmbedding(Part):
     kernel_libraries = ("embedding",)
 
     def __init__(self, vocab_size: int, hidden_size: int, weight_name: str = "weight",
-                 scale: float = 1.0, float32_stream: bool = False):
+                 scale: float = 1.0, float32_stream: bool = False, copies: int = 1):
         self.vocab_size, self.hidden_size = int(vocab_size), int(hidden_size)
         self.scale, self.float32_stream = float(scale), bool(float32_stream)
+        self.copies = int(copies)           # > 1: a row holds the result that many times (a model
+                                            # with several residual streams a token)
+        if self.copies != 1 and not self.float32_stream:
+            raise ValueError("several copies of the embedding are written into a float32 stream")
         if self.float32_stream:
             self.kernel_libraries = ("stream",)
         if self.scale != 1.0 and not self.float32_stream:
@@ -36,7 +40,7 @@ class TokenEmbedding(Part):
 
     def forward(self, token_ids: torch.Tensor) -> torch.Tensor:
         if self.float32_stream:
-            return ops.embedding_scaled(self.weight, token_ids, self.scale)
+            return ops.embedding_scaled(self.weight, token_ids, self.scale, self.copies)
         return ops.embedding(self.weight, token_ids)
 
 

@@ -18,9 +18,11 @@ class RMSNorm(Part):
     kernel_libraries = ("norm", "gemm", "gemm_rows", "stream")
     takes_pending_product = True
 
-    def __init__(self, size: int, eps: float, weight_name: str = "weight"):
+    def __init__(self, size: int, eps: float, weight_name: str = "weight", streams: int = 1):
         self.size = int(size)
         self.eps = float(eps)
+        self.streams = int(streams)         # > 1: the rows hold that many float32 streams side by
+                                            # side, and their sum is what is normed
         self.weight_name = weight_name
         self.weight: Optional[torch.Tensor] = None
         self.dtype: Optional[torch.dtype] = None
@@ -48,6 +50,10 @@ class RMSNorm(Part):
                                                     blocked=x.blocked)
                 return PendingScale(y, scale), residual
         x = as_tensor(x)
+        if self.streams > 1:
+            if residual is not None:
+                raise ValueError("a norm over the sum of several streams takes no residual")
+            return ops.hyper_mix(x, self.streams, None, None, None, None, self.weight, self.eps, self.dtype), x
         if residual is None and x.dtype == torch.float32 and self.dtype not in (None, torch.float32):
             # rows of a residual stream that is kept in float32: the result in the engine's dtype
             return ops.stream_rmsnorm(x, self.weight, self.eps, self.dtype), x

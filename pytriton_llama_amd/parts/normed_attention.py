@@ -32,6 +32,8 @@ class NormedAttention(Part):
                 heads, weights of that size; None: no norm), then rotation of the first rot_dims
                 entries of every head (entry i with i + rot_dims / 2) by position * frequency
         a_m = softmax_j<=i (q_m(i) . k_m(j) * scale) v(j)         one result a map, same values
+                (``window``: over the keys with i - j < window only, the query's own and the
+                window - 1 before it; pages that every later query has left behind are given back)
 
     maps = 1: out = W_o concat_h a + b_o.
     maps = 2 (differential attention: the second map is subtracted so that what both maps give
@@ -51,7 +53,7 @@ class NormedAttention(Part):
                  scale: Optional[float] = None, eps: float = 1e-6, qk_norm: Optional[str] = "head",
                  maps: int = 1, diff: float = 0.0, bias: bool = True, gated: bool = False,
                  rot_dims: int = 0, rot_base: float = 10000.0, rot_scaling: Optional[dict] = None,
-                 own_kv: bool = True, q_name: str = "q", k_name: str = "k", v_name: str = "v",
+                 own_kv: bool = True, window: Optional[int] = None, q_name: str = "q", k_name: str = "k", v_name: str = "v",
                  g_name: str = "g", o_name: str = "o", lambda_names=("lq1", "lk1", "lq2", "lk2")):
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} heads are not a multiple of {num_kv_heads} kv heads")
@@ -73,6 +75,9 @@ class NormedAttention(Part):
         self.norm_mode = {None: ops.NORM_NONE, "head": ops.NORM_HEAD, "whole": ops.NORM_WHOLE}[qk_norm]
         self.bias, self.gated, self.own_kv = bool(bias), bool(gated), bool(own_kv)
         self.rot_dims = int(rot_dims)
+        if window is not None and window <= 0:
+            raise ValueError("a window holds at least the query's own position")
+        self.window = int(window) if window else None
         self.mag = 1.0
         self.inv_freq_host = None
         if self.rot_dims:
@@ -119,16 +124,20 @@ class NormedAttention(Part):
         per_kv = self.num_heads // self.num_kv_heads
         base = max(1, n_dec * self.num_kv_heads * self.maps * (-(-per_kv // 4)))
         want = -(-2 * ops.compute_units(device) // base)
-        return max(1, min(want, -(-max(ctx.ctx_lens[:n_dec]) // turn), 64))
+        span = max(ctx.ctx_lens[:n_dec])
+        if self.window:
+            span = min(span, self.window)
+        return max(1, min(want, -(-span // turn), 64))
 
     def attend(self, a, q, cache, ctx, group) -> None:
         """Leading sequences of one token: the split-KV kernel; the rest: the matrix-core kernel in
         64-row blocks (bfloat16, sizes that are multiples of 32 up to 128) or the vector kernel in
         16-row blocks."""
         n_dec = ctx.num_decode_seqs if ops.attention_decode_kv_fits(self.dim, self.vdim) else 0
+        window = self.window or 0
         if n_dec:
             ops.attention_decode_kv(a, q, cache.k, cache.v, ctx.q_start, ctx.ctx_len, group.block_table, n_dec,
-                                    self.scale, self.maps, self.decode_splits(ctx, n_dec, q.device))
+                                    self.scale, self.maps, self.decode_splits(ctx, n_dec, q.device), window)
         if n_dec == ctx.num_seqs:
             return
         if n_dec == ctx.num_decode_seqs and ops.attention_prefill_mfma_kv_fits(
@@ -139,17 +148,18 @@ class NormedAttention(Part):
             t = max(1, held // (self.num_heads * self.maps))
             blocks = ws.numel()
             ops.attention_prefill_mfma_kv(a, q, cache.k, cache.v, ctx.q_start, ctx.ctx_len, group.block_table,
-                                          ws, wo, self.scale, self.maps, blocks if blocks <= 2 * t else t)
+                                          ws, wo, self.scale, self.maps, blocks if blocks <= 2 * t else t,
+                                          window)
             return
         ws, wo = ctx.work[PORTIONS_16 if n_dec else ALL_16]
         ops.attention_generic_kv(a, q, cache.k, cache.v, ctx.q_start, ctx.ctx_len, group.block_table,
-                                 ws, wo, self.scale, self.maps)
+                                 ws, wo, self.scale, self.maps, window)
 
     def cache_spec(self):
         if not self.own_kv:
             return None
         return PagedSpec((PagedTensor("k", (self.num_kv_heads * self.maps, self.dim), 1),
-                          PagedTensor("v", (self.num_kv_heads, self.vdim), 1)), None)
+                          PagedTensor("v", (self.num_kv_heads, self.vdim), 1)), self.window)
 
     def _norm_sizes(self):
         if self.norm_mode == ops.NORM_WHOLE:

@@ -174,6 +174,81 @@ class GatedDeltaRule(_MatrixStateMixer):
         return out
 
 
+@register_part("mixer", "selective_scan")
+class SelectiveScan(Part):
+    """The selective scan of Mamba (Gu, Dao: "Mamba: Linear-Time Sequence Modeling with Selective
+    State Spaces"): W_in x = [u | z] (``inner`` channels each); u passes a short causal
+    convolution over time ([inner, taps], the last tap is the current token's, with a bias) and
+    SiLU; W_x u = [r | B | C] (dt_rank, state, state entries); per channel c, with
+    dt = softplus(w_dt[c] . r + b_c) and A = -exp(A_log),
+
+        S[c, n] <- exp(dt A[c, n]) S[c, n] + dt u_c B_n;    y_c = sum_n S[c, n] C_n + D_c u_c
+
+    then y * silu(z) and W_o. S [inner, state] and the convolution's last taps - 1 inputs live in
+    the request's state slot in float32; the convolution, step sizes, decays and the recurrence are
+    float32 (the two first projections' results are taken in float32, W_dt is held in float32)."""
+    kernel_libraries = ("selective", "recurrent") + LINEAR_LIBRARIES
+
+    def __init__(self, hidden_size: int, inner: int, state: int, dt_rank: int, taps: int,
+                 in_name: str = "in", conv_name: str = "conv", conv_bias_name: str = "conv.b", x_name: str = "x",
+                 dt_name: str = "dt", dt_bias_name: str = "dt.b", A_log_name: str = "A_log", D_name: str = "D",
+                 o_name: str = "o"):
+        if state > 256:
+            raise ValueError(f"the scan kernel takes up to 256 states a channel, got {state}")
+        if taps < 1:
+            raise ValueError("a convolution has at least one tap")
+        self.hidden_size, self.inner, self.state = int(hidden_size), int(inner), int(state)
+        self.dt_rank, self.taps = int(dt_rank), int(taps)
+        self.names = dict(i=in_name, conv=conv_name, conv_b=conv_bias_name, x=x_name, dt=dt_name,
+                          dt_b=dt_bias_name, A_log=A_log_name, D=D_name, o=o_name)
+        self.tail_off = self.inner * self.state
+        self.w_in = self.w_x = self.o = self.w_in_blocked = self.w_x_blocked = self.o_blocked = None
+        self.conv_weight = self.conv_bias = self.w_dt = self.dt_bias = self.A_log = self.D = None
+
+    def cache_spec(self):
+        return StateSpec((ops.selective_state_floats(self.inner, self.state, self.taps),), torch.float32)
+
+    def param_sources(self) -> List[ParamSource]:
+        n, W, C, N, R = self.names, self.hidden_size, self.inner, self.state, self.dt_rank
+        return [ParamSource(n["i"], (2 * C, W)),
+                ParamSource(n["conv"], (C, self.taps), "vector", init=("normal", 0.0, 0.5)),
+                ParamSource(n["conv_b"], (C,), "vector", init=("normal", 0.0, 0.1)),
+                ParamSource(n["x"], (R + 2 * N, C)),
+                ParamSource(n["dt"], (C, R), "vector", init=("normal", 0.0, R ** -0.5)),
+                ParamSource(n["dt_b"], (C,), "vector", init=("uniform", -4.0, -1.0)),
+                ParamSource(n["A_log"], (C, N), "vector", init=("uniform", -1.0, 1.5)),
+                ParamSource(n["D"], (C,), "vector"),
+                ParamSource(n["o"], (W, C))]
+
+    def load(self, tensors, dtype, device) -> None:
+        n = self.names
+        self.w_in = place(tensors[n["i"]], "matrix", dtype, device)
+        self.w_x = place(pad_rows(tensors[n["x"]]), "matrix", dtype, device)
+        self.o = place(tensors[n["o"]], "matrix", dtype, device)
+        for attr, key in (("conv_weight", "conv"), ("conv_bias", "conv_b"), ("w_dt", "dt"), ("dt_bias", "dt_b"),
+                          ("A_log", "A_log"), ("D", "D")):
+            setattr(self, attr, place(tensors[n[key]], "vector", dtype, device))
+
+    def make_decode_copies(self) -> int:
+        self.w_in_blocked, self.w_x_blocked, self.o_blocked = (decode_copy(self.w_in), decode_copy(self.w_x),
+                                                               decode_copy(self.o))
+        return sum(t.numel() * t.element_size() for t in (self.w_in_blocked, self.w_x_blocked, self.o_blocked)
+                   if t is not None)
+
+    def forward(self, x, ctx, cache):
+        x = as_tensor(x)
+        C, N, R = self.inner, self.state, self.dt_rank
+        p = linear(x, self.w_in, out_dtype=torch.float32, blocked=self.w_in_blocked)
+        u, u_lp = ops.selective_conv(p, 0, self.conv_weight, self.conv_bias, cache.state, self.tail_off,
+                                     ctx.q_start, ctx.state_slots, ctx.max_q_len, x.dtype)
+        if self.taps > 1:
+            ops.conv_tail_update(p, 0, C, self.taps, cache.state, self.tail_off, ctx.q_start, ctx.state_slots)
+        r = linear(u if u_lp is None else u_lp, self.w_x, out_dtype=torch.float32, blocked=self.w_x_blocked)
+        y = ops.selective_scan(u, p, C, r, R, R, R + N, self.w_dt, self.dt_bias, self.A_log, self.D,
+                               cache.state, ctx.q_start, ctx.state_slots, x.dtype)
+        return linear(y, self.o, out_dtype=torch.float32, blocked=self.o_blocked)
+
+
 @register_part("mixer", "parallel")
 class ParallelMixers(Part):
     """Two mixers side by side on one input: left_scale * left(x) + right_scale * right(x). Each
