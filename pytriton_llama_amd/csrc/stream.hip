@@ -332,10 +332,10 @@ hyper_mix_kernel(float* __restrict__ streams, const TY* __restrict__ y, const fl
       float nx[SM];
 #pragma unroll
       for (int t = 0; t < SM; ++t) {
-        float a = co[t] * v;
+        float a = t < S ? co[t] * v : 0.f;         // (entries from S on are not there: never read)
 #pragma unroll
         for (int s = 0; s < SM; ++s) a = fmaf(s < S && t < S ? cm[s * S + t] : 0.f, x[s], a);
-        nx[t] = a;
+        nx[t] = t < S ? a : 0.f;
       }
 #pragma unroll
       for (int t = 0; t < SM; ++t) {

@@ -19,9 +19,13 @@ import torch
 # The dtype an engine rounds to where it stores a result between kernels; None: nothing is rounded.
 ROUND_TO = None
 
-# When a list: every routed feed-forward appends a tensor [T]: the gap between the choice score of
-# the last expert taken and the first one left out (a close call may go either way under rounding).
+# When a list: every routed feed-forward appends a bool tensor [T]: whether the choice between the
+# last expert taken and the first one left out is a close call that rounding may turn and that
+# matters. Rounding moves a score by a small share of itself, so the call is close when the gap
+# between the two choice scores is below CLOSE_CALL times the sum of the two scores; it matters
+# when the expert taken has more than a thousandth of the token's weight.
 ROUTER_MARGINS = None
+CLOSE_CALL = 0.1
 
 
 def stored(x):
@@ -138,11 +142,16 @@ def route(h, router, correction, top, scale):
     s = torch.softmax(lin(h, router), dim=-1)
     choice = s + correction
     idx = torch.topk(choice, top, dim=-1).indices
-    if ROUTER_MARGINS is not None:
-        srt = torch.sort(choice, dim=-1, descending=True).values
-        ROUTER_MARGINS.append(srt[:, top - 1] - srt[:, top] if srt.shape[1] > top
-                              else torch.full((h.shape[0],), float("inf"), dtype=h.dtype))
     picked = torch.gather(s, 1, idx)
+    if ROUTER_MARGINS is not None:
+        if s.shape[1] > top:
+            order = torch.sort(choice, dim=-1, descending=True)
+            last, nxt = order.indices[:, top - 1:top], order.indices[:, top:top + 1]
+            gap = (order.values[:, top - 1] - order.values[:, top])
+            s_last, s_next = torch.gather(s, 1, last)[:, 0], torch.gather(s, 1, nxt)[:, 0]
+            ROUTER_MARGINS.append((gap < CLOSE_CALL * (s_last + s_next)) & (s_last > 1e-3 * picked.sum(-1)))
+        else:
+            ROUTER_MARGINS.append(torch.zeros(h.shape[0], dtype=torch.bool))
     return idx, picked / (picked.sum(-1, keepdim=True) + 1e-20) * scale, s
 
 
