@@ -278,6 +278,37 @@ VIRUSUN_SIZES = {
 }
 
 
+def matusun_shape(width, layers, heads, kv_heads, dim, window, inner, state, dt_rank, experts, identity, top,
+                  expert_ff, shared_ff, streams, loop, vocab):
+    """A Matusun config.json of a real model's layer sizes: windowed attention and the selective
+    scan in turn, a routed feed-forward in every layer, ``loop`` = (start, stop, times)."""
+    attn = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5,
+            "mask": {"size": window}, "rot": {"base": 10000.0, "dims": dim}}
+    scan = {"inner": inner, "state": state, "dt_rank": dt_rank, "conv": 4}
+    moe = {"kind": "moe", "expert": {"ff": expert_ff}, "shared": {"ff": shared_ff},
+           "router": {"experts": experts, "identity": identity, "top": top, "scale": 1.0}}
+    out = [{"type": "attention", "mixer": attn, "mlp": moe} if i % 2 == 0 else
+           {"type": "mamba1", "mixer": scan, "mlp": moe} for i in range(layers)]
+    return {"architecture": "Matusun", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "layers": out,
+            "streams": streams, "loop": dict(zip(("start", "stop", "times"), loop)), "initializer_range": 0.02}
+
+
+# name -> (Matusun sizes, the Llama shape of equal width, as many layers as Matusun runs, equal heads
+# and as many hidden feed-forward units a token)
+MATUSUN_SIZES = {
+    "2048": (dict(width=2048, layers=6, heads=16, kv_heads=4, dim=128, window=1024, inner=4096, state=16,
+                  dt_rank=128, experts=16, identity=2, top=2, expert_ff=2048, shared_ff=4096, streams=4,
+                  loop=(2, 4, 2), vocab=32000),
+             dict(num_hidden_layers=8, hidden_size=2048, num_attention_heads=16, num_key_value_heads=4,
+                  head_dim=128, intermediate_size=8192, vocab_size=32000, tie_word_embeddings=False)),
+    "4096": (dict(width=4096, layers=4, heads=32, kv_heads=8, dim=128, window=2048, inner=8192, state=16,
+                  dt_rank=256, experts=32, identity=4, top=4, expert_ff=2048, shared_ff=6144, streams=4,
+                  loop=(0, 0, 1), vocab=32000),
+             dict(num_hidden_layers=4, hidden_size=4096, num_attention_heads=32, num_key_value_heads=8,
+                  head_dim=128, intermediate_size=14336, vocab_size=32000, tie_word_embeddings=False)),
+}
+
+
 def engine_rates(cfg, dtype, S, batch, steps, warmup):
     """Prefill of one S-token prompt (one step) and decode steps of ``batch`` requests behind
     S-token prompts, through the whole engine, for any architecture."""
@@ -369,6 +400,10 @@ def virusun_beside_llama(args):
     return beside_llama(args, "virusun", args.virusun, args.virusun_models, VIRUSUN_SIZES, virusun_shape)
 
 
+def matusun_beside_llama(args):
+    return beside_llama(args, "matusun", args.matusun, args.matusun_models, MATUSUN_SIZES, matusun_shape)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -408,6 +443,10 @@ def main():
                     help="the same for the Virusun design (sizes of: 2048, 4096)")
     ap.add_argument("--virusun-models", default="virusun,llama",
                     help="with --virusun: which of the two models to run (for profiles of one of them)")
+    ap.add_argument("--matusun", default="", metavar="SIZES",
+                    help="the same for the Matusun design (sizes of: 2048, 4096)")
+    ap.add_argument("--matusun-models", default="matusun,llama",
+                    help="with --matusun: which of the two models to run (for profiles of one of them)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU: this engine has no multi-GPU path, --gpus {args.gpus} is not run")
@@ -436,6 +475,8 @@ def main():
         return rubasun_beside_llama(args)
     if args.virusun:
         return virusun_beside_llama(args)
+    if args.matusun:
+        return matusun_beside_llama(args)
     if args.mixed:
         return mixed_workload(args, cfg, short)
     if args.like_reference:
