@@ -244,3 +244,237 @@ extern "C" int ptl_selective_scan(void* out, int out_dtype, const float* xc, con
   if (out_dtype == PTL_DTYPE_BF16) return launch_scan<bf16_t>(a, n_seqs, st);
   return PTL_ERR_ARG;
 }
+
+// ---------------------------------------------------------------------------
+// Long portions: segments walked side by side.
+//
+// The transition of a state is a scalar, S <- e S + b with e = exp(dt A), so over a segment of
+// tokens S_end = exp(A sum(dt)) S_start + E, where E is what the segment makes of a zero state.
+// Four kernels:
+//   dt:       the step sizes of all rows, dt[t, c] = softplus(w_dt[c, :] . r_t + b_c), as a tiled
+//             float32 product (64 rows x 64 channels a workgroup, 4 x 4 a thread);
+//   local:    every segment from a zero state: E [N][C] and sum(dt) [C] into the workspace;
+//   combine:  the sequences' segments one after the other: the start state of each, and the
+//             slot's state behind the last;
+//   final:    every segment again from its start state, with the read-out and the gate.
+// In local and final a lane holds one channel and all its N states in registers (N up to 32),
+// so a token's dt, x and z are read once a channel, rows of B and C are the same for the whole
+// wave, and no sum goes across lanes. Per token the arithmetic is that of the chain; the sums
+// over the states and over the tokens before a segment are taken in another order.
+// FAST: exp(dt A) as one hardware exponential of dt (A log2 e); used where the engine's dtype is
+// not float32.
+
+#define SEG_LOG2E 1.4426950408889634f
+
+__global__ void __launch_bounds__(256)
+selective_dt_kernel(float* __restrict__ dt, const float* __restrict__ r, long ldr,
+                    const float* __restrict__ w, const float* __restrict__ b, int T, int C, int R) {
+  __shared__ float rs[32][68];
+  __shared__ float ws[32][68];
+  const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
+  const int c0 = blockIdx.x * 64, t0 = blockIdx.y * 64;
+  float acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
+  for (int k0 = 0; k0 < R; k0 += 32) {
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int idx = tid + 256 * i, row = idx >> 5, k = idx & 31;
+      const bool kin = k0 + k < R;
+      rs[k][row] = (kin && t0 + row < T) ? r[(size_t)(t0 + row) * ldr + k0 + k] : 0.f;
+      ws[k][row] = (kin && c0 + row < C) ? w[(size_t)(c0 + row) * R + k0 + k] : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < 32; ++k) {
+      const float4 a = *reinterpret_cast<const float4*>(&rs[k][ty * 4]);
+      const float4 v = *reinterpret_cast<const float4*>(&ws[k][tx * 4]);
+      const float av[4] = {a.x, a.y, a.z, a.w}, vv[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(av[i], vv[j], acc[i][j]);
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int t = t0 + ty * 4 + i;
+    if (t >= T) continue;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int c = c0 + tx * 4 + j;
+      if (c < C) dt[(size_t)t * C + c] = softplus_f(acc[i][j] + b[c]);
+    }
+  }
+}
+
+// The workspace of segment g of sequence s: [N][C] states and [C] sums of dt.
+__device__ __forceinline__ size_t seg_work(int seq, int segments, int g, int C, int N) {
+  return (size_t)(seq * segments + g) * (size_t)(N + 1) * C;
+}
+
+// grid (blocks of 64 channels, segments, sequences), one wave a workgroup
+template <int NS, bool EXACT, bool FAST, bool FINAL, typename TO>
+__global__ void __launch_bounds__(64)
+selective_segment_kernel(TO* __restrict__ out, const float* __restrict__ dt, const float* __restrict__ xc,
+                         const float* __restrict__ z, long ldz, const float* __restrict__ r, long ldr,
+                         int b_off, int c_off, const float* __restrict__ A_log, const float* __restrict__ D,
+                         float* __restrict__ ends, const float* __restrict__ starts, int segments, int seg_len,
+                         const int32_t* __restrict__ q_start, int C, int N) {
+  const int seq = blockIdx.z, g = blockIdx.y;
+  const int row0 = q_start[seq];
+  const int qlen = q_start[seq + 1] - row0;
+  const int i0 = g * seg_len;
+  if (i0 >= qlen) return;
+  const int i1 = min(i0 + seg_len, qlen);
+  const int c = blockIdx.x * 64 + threadIdx.x;
+  const bool live = c < C;
+  const int cc = min(c, C - 1);            // (a lane past the end repeats the last channel; never stored)
+  const size_t wk = seg_work(seq, segments, g, C, N);
+  float A[NS], S[NS];
+#pragma unroll
+  for (int n = 0; n < NS; ++n) {
+    const bool in = EXACT || n < N;
+    A[n] = in ? -expf(A_log[(size_t)cc * N + n]) * (FAST ? SEG_LOG2E : 1.f) : 0.f;
+    S[n] = (FINAL && in) ? starts[wk + (size_t)n * C + cc] : 0.f;
+  }
+  const float Dc = D[cc];
+  float sum = 0.f;
+  size_t row = (size_t)(row0 + i0);
+  float d = dt[row * C + cc], x = xc[row * C + cc], zz = FINAL ? z[row * ldz + cc] : 0.f;
+  for (int i = i0; i < i1; ++i, ++row) {
+    const float dc = d, xv = x, zc = zz;
+    if (i + 1 < i1) {                      // the next token's, while this one is worked on
+      d = dt[(row + 1) * C + cc];
+      x = xc[(row + 1) * C + cc];
+      if (FINAL) zz = z[(row + 1) * ldz + cc];
+    }
+    const float* __restrict__ Bt = r + row * ldr + b_off;
+    const float* __restrict__ Ct = r + row * ldr + c_off;
+    const float dx = dc * xv;
+    float acc = 0.f;
+#pragma unroll
+    for (int n = 0; n < NS; ++n) {
+      if (EXACT || n < N) {
+        const float e = FAST ? __builtin_amdgcn_exp2f(dc * A[n]) : expf(dc * A[n]);
+        S[n] = fmaf(e, S[n], dx * Bt[n]);
+        if (FINAL) acc = fmaf(S[n], Ct[n], acc);
+      }
+    }
+    if (FINAL) {
+      if (live) out[row * C + c] = from_float<TO>(fmaf(Dc, xv, acc) * silu_f(zc));
+    } else {
+      sum += dc;
+    }
+  }
+  if (!FINAL && live) {
+#pragma unroll
+    for (int n = 0; n < NS; ++n)
+      if (EXACT || n < N) ends[wk + (size_t)n * C + c] = S[n];
+    ends[wk + (size_t)N * C + c] = sum;
+  }
+}
+
+// grid (blocks of 256 (state, channel) pairs, sequences): a thread takes one state of one channel
+// through the sequence's segments
+__global__ void __launch_bounds__(256)
+selective_combine_kernel(float* __restrict__ starts, const float* __restrict__ ends, float* __restrict__ state,
+                         long slot_stride, const float* __restrict__ A_log, int segments, int seg_len,
+                         const int32_t* __restrict__ q_start, const int32_t* __restrict__ state_slots, int C,
+                         int N) {
+  const int seq = blockIdx.y;
+  const int qlen = q_start[seq + 1] - q_start[seq];
+  if (qlen <= 0) return;
+  const int G = (qlen + seg_len - 1) / seg_len;
+  const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= (size_t)C * N) return;
+  const int n = (int)(idx / C), c = (int)(idx - (size_t)n * C);
+  float* st = state + (size_t)state_slots[seq] * slot_stride + (size_t)c * N + n;
+  const float A = -expf(A_log[(size_t)c * N + n]);
+  float S = *st;
+#pragma unroll 4
+  for (int g = 0; g < G; ++g) {
+    const size_t wk = seg_work(seq, segments, g, C, N);
+    const float E = ends[wk + (size_t)n * C + c];
+    const float sd = ends[wk + (size_t)N * C + c];
+    starts[wk + (size_t)n * C + c] = S;
+    S = fmaf(expf(A * sd), S, E);
+  }
+  *st = S;
+}
+
+struct SegLaunch {
+  void* out; const float* dt; const float* xc; const float* z; long ldz; const float* r; long ldr;
+  int b_off, c_off; const float* A_log; const float* D; float* ends; float* starts; int segments, seg_len;
+  const int32_t* q_start; int C, N, n_seqs;
+};
+
+template <int NS, bool EXACT, bool FAST, typename TO>
+static int launch_segments(const SegLaunch& a, bool final, hipStream_t st) {
+  dim3 grid((a.C + 63) / 64, a.segments, a.n_seqs);
+  if (final)
+    selective_segment_kernel<NS, EXACT, FAST, true, TO><<<grid, 64, 0, st>>>(
+        (TO*)a.out, a.dt, a.xc, a.z, a.ldz, a.r, a.ldr, a.b_off, a.c_off, a.A_log, a.D, a.ends, a.starts,
+        a.segments, a.seg_len, a.q_start, a.C, a.N);
+  else
+    selective_segment_kernel<NS, EXACT, FAST, false, TO><<<grid, 64, 0, st>>>(
+        (TO*)a.out, a.dt, a.xc, a.z, a.ldz, a.r, a.ldr, a.b_off, a.c_off, a.A_log, a.D, a.ends, a.starts,
+        a.segments, a.seg_len, a.q_start, a.C, a.N);
+  return ptl_launch_status();
+}
+
+template <bool FAST, typename TO>
+static int launch_segments_n(const SegLaunch& a, bool final, hipStream_t st) {
+  const int N = a.N;
+  if (N == 8) return launch_segments<8, true, FAST, TO>(a, final, st);
+  if (N == 16) return launch_segments<16, true, FAST, TO>(a, final, st);
+  if (N == 32) return launch_segments<32, true, FAST, TO>(a, final, st);
+  if (N < 8) return launch_segments<8, false, FAST, TO>(a, final, st);
+  if (N < 16) return launch_segments<16, false, FAST, TO>(a, final, st);
+  return launch_segments<32, false, FAST, TO>(a, final, st);
+}
+
+// The selective scan of a step with long portions. T rows in all; every sequence's rows are cut
+// into segments of seg_len tokens, at most ``segments`` a sequence. dt_work: T * C floats;
+// work: 2 * n_seqs * segments * (N + 1) * C floats. N up to 32.
+extern "C" int ptl_selective_scan_segments(void* out, int out_dtype, const float* xc, const float* z, long ldz,
+                                           const float* r, long ldr, int b_off, int c_off, const float* w_dt,
+                                           const float* dt_b, const float* A_log, const float* D, float* state,
+                                           long slot_stride, float* dt_work, float* work, int segments,
+                                           int seg_len, const int32_t* q_start, const int32_t* state_slots,
+                                           int n_seqs, int T, int C, int N, int R, int fast, hipStream_t st) {
+  if (n_seqs <= 0 || T <= 0) return PTL_OK;
+  if (C <= 0 || N <= 0 || N > 32 || R <= 0 || n_seqs > 65535 || segments <= 0 || segments > 65535 ||
+      seg_len <= 0 || (T + 63) / 64 > 65535)
+    return PTL_ERR_ARG;
+  {
+    dim3 grid((C + 63) / 64, (T + 63) / 64);
+    selective_dt_kernel<<<grid, 256, 0, st>>>(dt_work, r, ldr, w_dt, dt_b, T, C, R);
+    if (int e = ptl_launch_status()) return e;
+  }
+  float* ends = work;
+  float* starts = work + (size_t)n_seqs * segments * (size_t)(N + 1) * C;
+  SegLaunch a{out, dt_work, xc, z, ldz, r, ldr, b_off, c_off, A_log, D, ends, starts, segments, seg_len,
+              q_start, C, N, n_seqs};
+  for (int pass = 0; pass < 2; ++pass) {
+    int e;
+    if (out_dtype == PTL_DTYPE_F32)
+      e = fast ? launch_segments_n<true, float>(a, pass == 1, st) : launch_segments_n<false, float>(a, pass == 1, st);
+    else if (out_dtype == PTL_DTYPE_BF16)
+      e = fast ? launch_segments_n<true, bf16_t>(a, pass == 1, st)
+               : launch_segments_n<false, bf16_t>(a, pass == 1, st);
+    else
+      return PTL_ERR_ARG;
+    if (e) return e;
+    if (pass == 0) {
+      dim3 grid((unsigned)(((size_t)C * N + 255) / 256), n_seqs);
+      selective_combine_kernel<<<grid, 256, 0, st>>>(starts, ends, state, slot_stride, A_log, segments, seg_len,
+                                                     q_start, state_slots, C, N);
+      if (int e2 = ptl_launch_status()) return e2;
+    }
+  }
+  return PTL_OK;
+}

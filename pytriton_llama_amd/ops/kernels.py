@@ -1756,15 +1756,35 @@ def selective_conv(p: torch.Tensor, x_off: int, conv_weight: torch.Tensor, conv_
     return xc, lp
 
 
+SELECTIVE_SEGMENTS_FROM = 64      # rows of the longest sequence of a step from which segments are used
+SELECTIVE_SEGMENT_STATES = 32     # states a channel up to which a lane can hold them all
+SELECTIVE_SEGMENT_WAVES = 4096    # waves of a pass that fill the chip; segments are as long as this allows
+
+
+def selective_segment(n_seqs: int, max_q_len: int, channels: int) -> int:
+    """Tokens of a segment of a step's long portions: a power of two from 16 to 256, as long as the
+    step still has SELECTIVE_SEGMENT_WAVES waves (64 channels a wave and segment)."""
+    waves = max(1, n_seqs) * -(-channels // 64)
+    seg = 256
+    while seg > 16 and waves * -(-max_q_len // seg) < SELECTIVE_SEGMENT_WAVES:
+        seg //= 2
+    return seg
+
+
 def selective_scan(xc: torch.Tensor, p: torch.Tensor, z_off: int, r: torch.Tensor, rank: int, b_off: int,
                    c_off: int, w_dt: torch.Tensor, dt_bias: torch.Tensor, A_log: torch.Tensor, D: torch.Tensor,
                    state: torch.Tensor, q_start: torch.Tensor, state_slots: torch.Tensor,
-                   out_dtype: torch.dtype) -> torch.Tensor:
+                   out_dtype: torch.dtype, max_q_len: int = 0, seg_len: int = 0) -> torch.Tensor:
     """The recurrence S <- exp(dt A) S + dt x B, y = S C + D x, and the gate y * silu(z), for every
     sequence of the step from its slot's state [C, N] (at the start of the slot), which it leaves
     advanced. xc float32 [T, C]; z = p[:, z_off : z_off + C] (float32); r float32 rows with the
     step input in columns 0..rank-1, B [N] at b_off, C [N] at c_off; w_dt [C, rank], dt_bias [C],
-    A_log [C, N], D [C] float32. Returns [T, C] in ``out_dtype``."""
+    A_log [C, N], D [C] float32. Returns [T, C] in ``out_dtype``. ``max_q_len``: the rows of the
+    step's longest sequence (or a bound); from SELECTIVE_SEGMENTS_FROM rows on, with up to
+    SELECTIVE_SEGMENT_STATES states a channel, the sequences are worked on in segments side by side
+    (``seg_len`` tokens each, 0: chosen by selective_segment): the transition of a state is a
+    scalar, so a segment's start state follows from what the segments before it add to a zero state
+    and the sums of their step sizes."""
     _f32_rows(p, "selective_scan: p")
     _f32_rows(r, "selective_scan: r")
     _need_gpu(xc, w_dt, dt_bias, A_log, D, state, q_start, state_slots)
@@ -1792,6 +1812,21 @@ def selective_scan(xc: torch.Tensor, p: torch.Tensor, z_off: int, r: torch.Tenso
         raise KernelError("selective_scan: q_start has one entry more than there are sequences")
     out = torch.empty((T, C), dtype=out_dtype, device=xc.device)
     z = p[:, z_off:]
+    max_q_len = min(int(max_q_len), T)
+    if max_q_len >= SELECTIVE_SEGMENTS_FROM and N <= SELECTIVE_SEGMENT_STATES:
+        seg_len = int(seg_len) or selective_segment(n, max_q_len, C)
+        segments = -(-max_q_len // seg_len)
+        work_floats = 2 * n * segments * (N + 1) * C
+        if segments <= 65535 and work_floats <= (1 << 28) and T <= 64 * 65535:
+            dt_work = torch.empty((T, C), dtype=torch.float32, device=xc.device)
+            work = torch.empty((work_floats,), dtype=torch.float32, device=xc.device)
+            _check(library.load("selective").ptl_selective_scan_segments(
+                _ptr(out), _dtype_code(out), _ptr(xc), _ptr(z), ctypes.c_long(p.stride(0)), _ptr(r),
+                ctypes.c_long(r.stride(0)), int(b_off), int(c_off), _ptr(w_dt), _ptr(dt_bias), _ptr(A_log),
+                _ptr(D), _ptr(state), ctypes.c_long(state.stride(0)), _ptr(dt_work), _ptr(work), int(segments),
+                int(seg_len), _ptr(q_start), _ptr(state_slots), n, T, C, N, R,
+                0 if out_dtype == torch.float32 else 1, _stream()), "selective_scan")
+            return out
     _check(library.load("selective").ptl_selective_scan(
         _ptr(out), _dtype_code(out), _ptr(xc), _ptr(z), ctypes.c_long(p.stride(0)), _ptr(r),
         ctypes.c_long(r.stride(0)), int(b_off), int(c_off), _ptr(w_dt), _ptr(dt_bias), _ptr(A_log), _ptr(D),

@@ -245,7 +245,7 @@ class SelectiveScan(Part):
             ops.conv_tail_update(p, 0, C, self.taps, cache.state, self.tail_off, ctx.q_start, ctx.state_slots)
         r = linear(u if u_lp is None else u_lp, self.w_x, out_dtype=torch.float32, blocked=self.w_x_blocked)
         y = ops.selective_scan(u, p, C, r, R, R, R + N, self.w_dt, self.dt_bias, self.A_log, self.D,
-                               cache.state, ctx.q_start, ctx.state_slots, x.dtype)
+                               cache.state, ctx.q_start, ctx.state_slots, x.dtype, ctx.max_q_len)
         return linear(y, self.o, out_dtype=torch.float32, blocked=self.o_blocked)
 
 

@@ -127,6 +127,69 @@ def test_selective_scan_in_portions_and_batches(gpu_device, C, N, R, taps):
             assert float((g - w).abs().max()) < 3e-5 * float(w.abs().max()), sizes
 
 
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("C,N,R,taps,seg", [(64, 16, 4, 4, 16), (40, 8, 3, 3, 32), (70, 20, 5, 2, 0), (130, 32, 9, 1, 64),
+                                            (33, 5, 2, 3, 16), (24, 12, 40, 4, 0)])
+def test_selective_scan_of_long_portions_in_segments(gpu_device, C, N, R, taps, seg, out_dtype):
+    """Sequences of unequal lengths whose long portions are walked in segments side by side
+    (portions that end inside a segment, at its end and one token behind it; a sequence of one
+    token beside them; short portions of the same sequences through the chain before and after),
+    against the recurrence written out; the state that the segments leave is the one that single
+    tokens go on from."""
+    from pytriton_llama_amd import ops
+    torch.manual_seed(C * N + R)
+    lens = [333, 1, 129, 200]
+    slots = [1, 4, 0, 2]
+    f64 = torch.float64
+    cw, cb = 0.5 * torch.randn(C, taps, dtype=f64), 0.1 * torch.randn(C, dtype=f64)
+    w_dt, dt_b = torch.randn(C, R, dtype=f64) / R ** 0.5, torch.rand(C, dtype=f64) * 3 - 4
+    A_log, D = torch.rand(C, N, dtype=f64) * 2.5 - 1, torch.randn(C, dtype=f64)
+    ps = [torch.randn(n, 2 * C, dtype=f64) for n in lens]
+    rs = [torch.randn(n, R + 2 * N, dtype=f64) for n in lens]
+    want = []
+    for p, r in zip(ps, rs):
+        u = pm.silu(pm.causal_conv(p[:, :C], cw, cb))
+        dt = pm.softplus(r[:, :R] @ w_dt.T + dt_b)
+        y = pm.selective_scan(u, dt, -torch.exp(A_log), r[:, R:R + N], r[:, R + N:R + 2 * N], D)
+        want.append(y * pm.silu(p[:, C:]))
+    tail_off = C * N
+    state = torch.randn(5, ops.selective_state_floats(C, N, taps), device="cuda")
+    args = [dev(t) for t in (cw, cb, w_dt, dt_b, A_log, D)]
+    tol = 3e-5 if out_dtype == torch.float32 else 1e-2
+    for sizes in ((400,), (3, 64, 1, 65, 2, 128, 1, 1, 100), (96, 1, 97)):
+        for s_ in slots:
+            state[s_].zero_()
+        got = [torch.zeros(n, C, dtype=f64) for n in lens]
+        cuts = [cut(n, sizes[i:] + sizes[:i]) for i, n in enumerate(lens)]
+        for step in range(max(len(c) for c in cuts)):
+            live = [i for i in range(len(lens)) if step < len(cuts[i])]
+            rows_p = torch.cat([ps[i][cuts[i][step][0]:cuts[i][step][1]] for i in live])
+            rows_r = torch.cat([rs[i][cuts[i][step][0]:cuts[i][step][1]] for i in live])
+            qlens = [cuts[i][step][1] - cuts[i][step][0] for i in live]
+            q_start = i32([0] + torch.tensor(qlens).cumsum(0).tolist())
+            sl = i32([slots[i] for i in live])
+            p_dev, r_dev = dev(rows_p), dev(rows_r)
+            u, _ = ops.selective_conv(p_dev, 0, args[0], args[1], state, tail_off, q_start, sl, max(qlens))
+            if taps > 1:
+                ops.conv_tail_update(p_dev, 0, C, taps, state, tail_off, q_start, sl)
+            y = ops.selective_scan(u, p_dev, C, r_dev, R, R, R + N, args[2], args[3], args[4], args[5],
+                                   state, q_start, sl, out_dtype, max(qlens), seg).double().cpu()
+            at = 0
+            for i, n in zip(live, qlens):
+                got[i][cuts[i][step][0]:cuts[i][step][1]] = y[at:at + n]
+                at += n
+        for g, w in zip(got, want):
+            assert float((g - w).abs().max()) < tol * float(w.abs().max()), sizes
+
+
+def test_segment_length_fills_the_chip():
+    from pytriton_llama_amd import ops
+    assert ops.selective_segment(1, 2048, 4096) == 32
+    assert ops.selective_segment(8, 2048, 4096) == 256
+    assert ops.selective_segment(1, 64, 64) == 16
+    assert ops.selective_segment(1, 1 << 20, 8192) == 256
+
+
 # ---- the router and the experts -----------------------------------------------------------------
 @pytest.mark.parametrize("E,ident,top,shared", [(5, 2, 3, True), (4, 0, 1, False), (2, 1, 3, True), (70, 3, 4, False),
                                                 (1, 1, 1, False)])
