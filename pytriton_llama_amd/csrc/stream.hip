@@ -303,11 +303,11 @@ extern "C" int ptl_gelu_gather_mul(void* out, const void* z, const void* table, 
 // from the (new) streams and normed into ``out``. Either half may be absent. Null coefficients
 // stand for a single plain stream: in = ones, mix = the identity, out = ones (then S = 1 is the
 // residual sum in front of a norm, and in = ones alone is the sum of the streams). One workgroup
-// a token; u waits in LDS between the pass that makes it and the one that scales it.
+// a token (of 1,024 threads when the rows are few, else 256); u waits in LDS between the pass that makes it and the one that scales it.
 #define HYPER_MAX_S 16
 
-template <int SM, typename TY, typename TO>
-__global__ void __launch_bounds__(256)
+template <int SM, int NT, typename TY, typename TO>
+__global__ void __launch_bounds__(NT)
 hyper_mix_kernel(float* __restrict__ streams, const TY* __restrict__ y, const float* __restrict__ mix,
                  const float* __restrict__ outc, const float* __restrict__ inc, const float* __restrict__ nw,
                  float eps, TO* __restrict__ out, int S, int H) {
@@ -323,7 +323,7 @@ hyper_mix_kernel(float* __restrict__ streams, const TY* __restrict__ y, const fl
   __syncthreads();
   float* row = streams + (size_t)blockIdx.x * S * H;
   float ss = 0.f;
-  for (int c = tid; c < H; c += 256) {
+  for (int c = tid; c < H; c += NT) {
     float x[SM];
 #pragma unroll
     for (int s = 0; s < SM; ++s) x[s] = s < S ? row[(size_t)s * H + c] : 0.f;
@@ -354,21 +354,29 @@ hyper_mix_kernel(float* __restrict__ streams, const TY* __restrict__ y, const fl
   if (!nw) return;
   ss = block_sum(ss, scratch);
   const float r = 1.0f / sqrtf(ss / (float)H + eps);
-  for (int c = tid; c < H; c += 256) out[(size_t)blockIdx.x * H + c] = from_float<TO>(us[c] * r * nw[c]);
+  for (int c = tid; c < H; c += NT) out[(size_t)blockIdx.x * H + c] = from_float<TO>(us[c] * r * nw[c]);
 }
 
 template <typename TY, typename TO>
 static int launch_hyper(float* streams, const void* y, const float* mix, const float* outc, const float* inc,
                         const float* nw, float eps, void* out, int T_, int S, int H, hipStream_t st) {
   const size_t lds = nw ? (size_t)H * sizeof(float) : 0;
+  // few rows: a row's entries over 1,024 threads, so that a thread's loads are one or two deep
+  const bool few = T_ <= 512 && H > 256;
 #define GO(SM)                                                                                       \
   {                                                                                                  \
     if (lds > 48 * 1024 &&                                                                           \
-        hipFuncSetAttribute((const void*)hyper_mix_kernel<SM, TY, TO>,                               \
-                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)     \
+        (hipFuncSetAttribute((const void*)hyper_mix_kernel<SM, 256, TY, TO>,                         \
+                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess ||  \
+         hipFuncSetAttribute((const void*)hyper_mix_kernel<SM, 1024, TY, TO>,                        \
+                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess))   \
       return PTL_ERR_LAUNCH;                                                                         \
-    hyper_mix_kernel<SM, TY, TO><<<T_, 256, lds, st>>>(streams, (const TY*)y, mix, outc, inc, nw, eps, \
-                                                       (TO*)out, S, H);                              \
+    if (few)                                                                                         \
+      hyper_mix_kernel<SM, 1024, TY, TO><<<T_, 1024, lds, st>>>(streams, (const TY*)y, mix, outc, inc, nw, \
+                                                                eps, (TO*)out, S, H);                \
+    else                                                                                             \
+      hyper_mix_kernel<SM, 256, TY, TO><<<T_, 256, lds, st>>>(streams, (const TY*)y, mix, outc, inc, nw,   \
+                                                              eps, (TO*)out, S, H);                  \
     return ptl_launch_status();                                                                      \
   }
   if (S <= 1) GO(1)

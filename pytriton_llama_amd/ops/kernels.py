@@ -1761,12 +1761,15 @@ SELECTIVE_SEGMENT_STATES = 32     # states a channel up to which a lane can hold
 SELECTIVE_SEGMENT_WAVES = 4096    # waves of a pass that fill the chip; segments are as long as this allows
 
 
-def selective_segment(n_seqs: int, max_q_len: int, channels: int) -> int:
+def selective_segment(n_seqs: int, max_q_len: int, channels: int, rows: int = 0) -> int:
     """Tokens of a segment of a step's long portions: a power of two from 16 to 256, as long as the
-    step still has SELECTIVE_SEGMENT_WAVES waves (64 channels a wave and segment)."""
-    waves = max(1, n_seqs) * -(-channels // 64)
+    step still has SELECTIVE_SEGMENT_WAVES waves (64 channels a wave and segment). ``rows``: the
+    rows of the step when known (a long portion beside single tokens has far fewer segments than
+    sequences times the longest one's)."""
+    n_seqs = max(1, int(n_seqs))
+    rows = min(int(rows), n_seqs * int(max_q_len)) if rows > 0 else n_seqs * int(max_q_len)
     seg = 256
-    while seg > 16 and waves * -(-max_q_len // seg) < SELECTIVE_SEGMENT_WAVES:
+    while seg > 16 and -(-channels // 64) * (rows // seg + n_seqs) < SELECTIVE_SEGMENT_WAVES:
         seg //= 2
     return seg
 
@@ -1814,7 +1817,7 @@ def selective_scan(xc: torch.Tensor, p: torch.Tensor, z_off: int, r: torch.Tenso
     z = p[:, z_off:]
     max_q_len = min(int(max_q_len), T)
     if max_q_len >= SELECTIVE_SEGMENTS_FROM and N <= SELECTIVE_SEGMENT_STATES:
-        seg_len = int(seg_len) or selective_segment(n, max_q_len, C)
+        seg_len = int(seg_len) or selective_segment(n, max_q_len, C, T)
         segments = -(-max_q_len // seg_len)
         work_floats = 2 * n * segments * (N + 1) * C
         if segments <= 65535 and work_floats <= (1 << 28) and T <= 64 * 65535:
