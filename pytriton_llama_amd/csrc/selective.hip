@@ -56,6 +56,33 @@ selective_conv_kernel(float* __restrict__ xc, TO* __restrict__ xc_lp, const floa
   const float* tail = state + (size_t)state_slots[seq] * slot_stride + tail_off;
   const float bias = cb ? cb[c] : 0.f;
   const int i1 = min(i0 + SCHUNK, qlen);
+  if (taps <= 8) {
+    // the last inputs stay in registers, the newest in the last place and the taps aligned to it, so
+    // that every input is read once (and taps - 1 before the block's first row)
+    float wv[8], win[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int k = j - (8 - taps);        // the tap in place j
+      wv[j] = k >= 0 ? cw[(size_t)c * taps + k] : 0.f;
+      win[j] = 0.f;
+      if (k >= 0 && j < 7) {
+        const int r = i0 - (taps - 1) + k;
+        win[j] = r >= 0 ? p[(size_t)(row0 + r) * ldp + x_off + c] : tail[(size_t)(taps - 1 + r) * C + c];
+      }
+    }
+    for (int i = i0; i < i1; ++i) {
+      win[7] = p[(size_t)(row0 + i) * ldp + x_off + c];
+      float s = bias;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) s = fmaf(wv[j], win[j], s);
+#pragma unroll
+      for (int j = 0; j < 7; ++j) win[j] = win[j + 1];
+      const float v = silu_f(s);
+      xc[(size_t)(row0 + i) * C + c] = v;
+      if (xc_lp) xc_lp[(size_t)(row0 + i) * C + c] = from_float<TO>(v);
+    }
+    return;
+  }
   for (int i = i0; i < i1; ++i) {
     float s = bias;
     for (int j = 0; j < taps; ++j) {
@@ -251,8 +278,8 @@ extern "C" int ptl_selective_scan(void* out, int out_dtype, const float* xc, con
 // The transition of a state is a scalar, S <- e S + b with e = exp(dt A), so over a segment of
 // tokens S_end = exp(A sum(dt)) S_start + E, where E is what the segment makes of a zero state.
 // Four kernels:
-//   dt:       the step sizes of all rows, dt[t, c] = softplus(w_dt[c, :] . r_t + b_c), as a tiled
-//             float32 product (64 rows x 64 channels a workgroup, 4 x 4 a thread);
+//   dt:       the step sizes of all rows, dt[t, c] = softplus(w_dt[c, :] . r_t + b_c), as a float32
+//             product on the matrix cores (64 rows x 128 channels a workgroup);
 //   local:    every segment from a zero state: E [N][C] and sum(dt) [C] into the workspace;
 //   combine:  the sequences' segments one after the other: the start state of each, and the
 //             slot's state behind the last;
@@ -261,53 +288,70 @@ extern "C" int ptl_selective_scan(void* out, int out_dtype, const float* xc, con
 // so a token's dt, x and z are read once a channel, rows of B and C are the same for the whole
 // wave, and no sum goes across lanes. Per token the arithmetic is that of the chain; the sums
 // over the states and over the tokens before a segment are taken in another order.
-// FAST: exp(dt A) as one hardware exponential of dt (A log2 e); used where the engine's dtype is
-// not float32.
+// FAST: exp(dt A) as one hardware exponential of dt (A log2 e), and the softplus from the
+// hardware's exponential and logarithm; used where the engine's dtype is not float32.
 
 #define SEG_LOG2E 1.4426950408889634f
 
+typedef float seg_f32x16 __attribute__((ext_vector_type(16)));
+
+// softplus from the hardware's exponential and logarithm (a step size below 1e-7 comes out as 0)
+__device__ __forceinline__ float softplus_fast(float x) { return x > 20.f ? x : __logf(1.0f + __expf(x)); }
+
+// dt[t, c] = softplus(b[c] + sum_k w[c, k] r[t, k]) on the matrix cores in float32
+// (v_mfma_f32_32x32x2_f32: float32 operands and sums). A wave takes 32 rows x 64 channels, a
+// workgroup of four waves 64 x 128. Of a block of 8 k, lane l holds r[t0 + l % 32][4 (l / 32) ..+3]
+// and the same entries of two rows of w; product m of the four takes entry m of every lane, so both
+// operands see the same k in the same place. VEC: rows of r and w allow 16-byte loads.
+template <bool VEC, bool FAST>
 __global__ void __launch_bounds__(256)
 selective_dt_kernel(float* __restrict__ dt, const float* __restrict__ r, long ldr,
                     const float* __restrict__ w, const float* __restrict__ b, int T, int C, int R) {
-  __shared__ float rs[32][68];
-  __shared__ float ws[32][68];
-  const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
-  const int c0 = blockIdx.x * 64, t0 = blockIdx.y * 64;
-  float acc[4][4];
+  const int wave = threadIdx.x >> 6, l = threadIdx.x & 63;
+  const int t0 = blockIdx.y * 64 + (wave >> 1) * 32, c0 = blockIdx.x * 128 + (wave & 1) * 64;
+  if (t0 >= T || c0 >= C) return;
+  const int j = l & 31, h = l >> 5;
+  const float* rp = r + (size_t)min(t0 + j, T - 1) * ldr;
+  const float* w0 = w + (size_t)min(c0 + j, C - 1) * R;
+  const float* w1 = w + (size_t)min(c0 + 32 + j, C - 1) * R;
+  seg_f32x16 acc0, acc1;
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int v = 0; v < 16; ++v) acc0[v] = acc1[v] = 0.f;
+#pragma unroll 4
+  for (int k0 = 0; k0 < R; k0 += 8) {
+    const int k = k0 + 4 * h;
+    float av[4], b0[4], b1[4];
+    if (VEC && k0 + 8 <= R) {
+      const float4 x = *reinterpret_cast<const float4*>(rp + k);
+      const float4 y0 = *reinterpret_cast<const float4*>(w0 + k);
+      const float4 y1 = *reinterpret_cast<const float4*>(w1 + k);
+      av[0] = x.x; av[1] = x.y; av[2] = x.z; av[3] = x.w;
+      b0[0] = y0.x; b0[1] = y0.y; b0[2] = y0.z; b0[3] = y0.w;
+      b1[0] = y1.x; b1[1] = y1.y; b1[2] = y1.z; b1[3] = y1.w;
+    } else {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
-  for (int k0 = 0; k0 < R; k0 += 32) {
-    __syncthreads();
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const int idx = tid + 256 * i, row = idx >> 5, k = idx & 31;
-      const bool kin = k0 + k < R;
-      rs[k][row] = (kin && t0 + row < T) ? r[(size_t)(t0 + row) * ldr + k0 + k] : 0.f;
-      ws[k][row] = (kin && c0 + row < C) ? w[(size_t)(c0 + row) * R + k0 + k] : 0.f;
+      for (int m = 0; m < 4; ++m) {
+        const bool in = k + m < R;
+        av[m] = in ? rp[k + m] : 0.f;
+        b0[m] = in ? w0[k + m] : 0.f;
+        b1[m] = in ? w1[k + m] : 0.f;
+      }
     }
-    __syncthreads();
 #pragma unroll
-    for (int k = 0; k < 32; ++k) {
-      const float4 a = *reinterpret_cast<const float4*>(&rs[k][ty * 4]);
-      const float4 v = *reinterpret_cast<const float4*>(&ws[k][tx * 4]);
-      const float av[4] = {a.x, a.y, a.z, a.w}, vv[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(av[i], vv[j], acc[i][j]);
+    for (int m = 0; m < 4; ++m) {
+      acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(av[m], b0[m], acc0, 0, 0, 0);
+      acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(av[m], b1[m], acc1, 0, 0, 0);
     }
   }
+  // entry v of a lane: row 8 (v / 4) + 4 (l / 32) + v % 4 of the tile, column l % 32
+  const int ca = c0 + j, cb = c0 + 32 + j;
+  const float ba = ca < C ? b[ca] : 0.f, bb = cb < C ? b[cb] : 0.f;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int t = t0 + ty * 4 + i;
+  for (int v = 0; v < 16; ++v) {
+    const int t = t0 + 8 * (v >> 2) + 4 * h + (v & 3);
     if (t >= T) continue;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int c = c0 + tx * 4 + j;
-      if (c < C) dt[(size_t)t * C + c] = softplus_f(acc[i][j] + b[c]);
-    }
+    if (ca < C) dt[(size_t)t * C + ca] = FAST ? softplus_fast(acc0[v] + ba) : softplus_f(acc0[v] + ba);
+    if (cb < C) dt[(size_t)t * C + cb] = FAST ? softplus_fast(acc1[v] + bb) : softplus_f(acc1[v] + bb);
   }
 }
 
@@ -451,8 +495,16 @@ extern "C" int ptl_selective_scan_segments(void* out, int out_dtype, const float
       seg_len <= 0 || (T + 63) / 64 > 65535)
     return PTL_ERR_ARG;
   {
-    dim3 grid((C + 63) / 64, (T + 63) / 64);
-    selective_dt_kernel<<<grid, 256, 0, st>>>(dt_work, r, ldr, w_dt, dt_b, T, C, R);
+    dim3 grid((C + 127) / 128, (T + 63) / 64);
+    const bool vec = R % 4 == 0 && ldr % 4 == 0 && ((uintptr_t)r & 15) == 0 && ((uintptr_t)w_dt & 15) == 0;
+    if (vec && fast)
+      selective_dt_kernel<true, true><<<grid, 256, 0, st>>>(dt_work, r, ldr, w_dt, dt_b, T, C, R);
+    else if (vec)
+      selective_dt_kernel<true, false><<<grid, 256, 0, st>>>(dt_work, r, ldr, w_dt, dt_b, T, C, R);
+    else if (fast)
+      selective_dt_kernel<false, true><<<grid, 256, 0, st>>>(dt_work, r, ldr, w_dt, dt_b, T, C, R);
+    else
+      selective_dt_kernel<false, false><<<grid, 256, 0, st>>>(dt_work, r, ldr, w_dt, dt_b, T, C, R);
     if (int e = ptl_launch_status()) return e;
   }
   float* ends = work;

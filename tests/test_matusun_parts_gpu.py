@@ -75,7 +75,7 @@ def cut(total, sizes):
     return out
 
 
-@pytest.mark.parametrize("C,N,R,taps", [(16, 16, 4, 4), (40, 8, 3, 3), (50, 20, 5, 1), (33, 40, 2, 2), (24, 130, 7, 4),
+@pytest.mark.parametrize("C,N,R,taps", [(16, 16, 4, 4), (40, 8, 3, 3), (50, 20, 5, 1), (33, 40, 2, 2), (24, 130, 7, 4), (20, 8, 3, 9),
                                         (130, 12, 20, 5)])
 def test_selective_scan_in_portions_and_batches(gpu_device, C, N, R, taps):
     """Three sequences advanced together in portions of changing sizes (down to one token, their
