@@ -110,32 +110,47 @@ class NormedAttention(Part):
     def work_lists(self):
         return (ALL_16, PORTIONS_16, PORTIONS_64)
 
-    def decode_splits(self, ctx, n_dec: int, device) -> int:
+    def decode_splits(self, ctx, n_dec: int, device, matrix_cores: bool = False) -> int:
         """How many workgroups share one decoding sequence's keys: enough to fill the compute
         units about twice over (measured on MI355X at batch 1 to 64 behind 2,048 keys: beyond that the
         merging of a workgroup's key slots costs more than the shorter loops save), never finer
-        than one turn of a workgroup."""
+        than one turn of a workgroup. ``matrix_cores``: for the matrix-core form (a workgroup a kv
+        head, 128 keys a turn; no splits once the batch brings 1.75 workgroups a compute unit)."""
         if self.force_decode_splits:
             return self.force_decode_splits
+        span = max(ctx.ctx_lens[:n_dec])
+        if self.window:
+            span = min(span, self.window)
+        cus = ops.compute_units(device)
+        if matrix_cores:
+            base = max(1, n_dec * self.num_kv_heads)
+            want = 1 if 4 * base >= 7 * cus else -(-2 * cus // base)
+            return max(1, min(want, -(-span // 128), 64))
         lpk = 1
         while lpk * 16 < max(self.dim, self.vdim):
             lpk <<= 1
         turn = 2 * (256 // lpk)
         per_kv = self.num_heads // self.num_kv_heads
         base = max(1, n_dec * self.num_kv_heads * self.maps * (-(-per_kv // 4)))
-        want = -(-2 * ops.compute_units(device) // base)
-        span = max(ctx.ctx_lens[:n_dec])
-        if self.window:
-            span = min(span, self.window)
+        want = -(-2 * cus // base)
         return max(1, min(want, -(-span // turn), 64))
 
     def attend(self, a, q, cache, ctx, group) -> None:
-        """Leading sequences of one token: the split-KV kernel; the rest: the matrix-core kernel in
+        """Leading sequences of one token: the split-KV kernel (its matrix-core form where one
+        map reads keys and values of one size that it takes); the rest: the matrix-core kernel in
         64-row blocks (bfloat16, sizes that are multiples of 32 up to 128) or the vector kernel in
         16-row blocks."""
         n_dec = ctx.num_decode_seqs if ops.attention_decode_kv_fits(self.dim, self.vdim) else 0
         window = self.window or 0
-        if n_dec:
+        # one map and keys as large as values: the matrix-core form of the split-KV kernel takes them
+        mfma = (n_dec and self.maps == 1 and self.dim == self.vdim and q.stride(0) % 8 == 0
+                and ops.attention_decode_mfma_fits(q.dtype, self.num_heads, self.num_kv_heads, self.dim,
+                                                   cache.page_size))
+        if mfma:
+            ops.attention_decode(a, q, cache.k, cache.v, ctx.q_start, ctx.ctx_len, group.block_table, n_dec,
+                                 self.scale, window, self.decode_splits(ctx, n_dec, q.device, True),
+                                 matrix_cores=True)
+        elif n_dec:
             ops.attention_decode_kv(a, q, cache.k, cache.v, ctx.q_start, ctx.ctx_len, group.block_table, n_dec,
                                     self.scale, self.maps, self.decode_splits(ctx, n_dec, q.device), window)
         if n_dec == ctx.num_seqs:
