@@ -130,18 +130,22 @@ struct SelArgs {
   float* state; long slot_stride;
   const int32_t* q_start; const int32_t* state_slots;
   int C, N, R;
+  int chunk;                     // tokens that go through LDS at a time: 1 to SCHUNK
 };
 
-// LDS of a workgroup, in floats: rows [SCHUNK][R + 2 N] | w_dt [16][R] | x, z, dt, y [SCHUNK][16] each
-static inline size_t scan_lds_floats(int N, int R) { return (size_t)SCHUNK * (R + 2 * N) + 16 * R + 4 * SCHUNK * 16; }
+// LDS of a workgroup, in floats: rows [chunk][R + 2 N] | w_dt [16][R] | x, z, dt, y [SCHUNK][16] each
+static inline size_t scan_lds_floats(int N, int R, int chunk) {
+  return (size_t)chunk * (R + 2 * N) + 16 * R + 4 * SCHUNK * 16;
+}
 
 template <int NPL, typename TO>
 __global__ void __launch_bounds__(256) selective_scan_kernel(SelArgs a) {
   extern __shared__ float lds[];
   const int N = a.N, R = a.R, C = a.C;
   const int RW = R + 2 * N;
-  float* rows = lds;                       // [SCHUNK][RW]: r | B | C of the chunk's tokens
-  float* wdt = rows + SCHUNK * RW;         // [16][R]
+  const int CH = a.chunk;
+  float* rows = lds;                       // [CH][RW]: r | B | C of the chunk's tokens
+  float* wdt = rows + CH * RW;             // [16][R]
   float* xs = wdt + 16 * R;                // [SCHUNK][16]
   float* zs = xs + SCHUNK * 16;
   float* dts = zs + SCHUNK * 16;
@@ -171,8 +175,9 @@ __global__ void __launch_bounds__(256) selective_scan_kernel(SelArgs a) {
   // the thread that computes the step size of (token tid >> 4, channel tid & 15)
   const int dch = min(c0 + (tid & 15), C - 1);
   const float dtb = a.dt_b[dch];
-  for (int t0 = 0; t0 < qlen; t0 += SCHUNK) {
-    const int nt = min(SCHUNK, qlen - t0);
+  const float dtb_own = a.dt_b[c];         // of the channel this thread walks
+  for (int t0 = 0; t0 < qlen; t0 += CH) {
+    const int nt = min(CH, qlen - t0);
     __syncthreads();                       // the chunk before is done with
     for (int i = tid; i < nt * RW; i += 256) {
       const int t = i / RW, k = i - t * RW;
@@ -187,7 +192,17 @@ __global__ void __launch_bounds__(256) selective_scan_kernel(SelArgs a) {
       }
     }
     __syncthreads();
-    {
+    if (nt <= 4) {
+      // few tokens: the 16 lanes of a channel share a token's sum
+      for (int t = 0; t < nt; ++t) {
+        const float* rr = rows + t * RW;
+        const float* ww = wdt + cg * R;
+        float s = 0.f;
+        for (int k = l; k < R; k += 16) s = fmaf(ww[k], rr[k], s);
+        s = row16_sum(s);
+        if (l == 0) dts[t * 16 + cg] = softplus_f(s + dtb_own);
+      }
+    } else {
       const int t = tid >> 4, ch = tid & 15;
       if (t < nt) {
         float s = dtb;
@@ -234,7 +249,7 @@ __global__ void __launch_bounds__(256) selective_scan_kernel(SelArgs a) {
 template <typename TO>
 static int launch_scan(const SelArgs& a, int n_seqs, hipStream_t st) {
   const int N = a.N;
-  const size_t lds = scan_lds_floats(N, a.R) * sizeof(float);
+  const size_t lds = scan_lds_floats(N, a.R, a.chunk) * sizeof(float);
   dim3 grid((a.C + 15) / 16, n_seqs);
 #define GO(NPL)                                                                                      \
   {                                                                                                  \
@@ -255,18 +270,21 @@ static int launch_scan(const SelArgs& a, int n_seqs, hipStream_t st) {
 
 // out [T, C] (engine dtype) from xc [T, C], z (float32, row stride ldz), the float32 rows r | B | C
 // (row stride ldr; r from column 0, B from b_off, C from c_off), w_dt [C, R], dt_b [C], A_log [C, N],
-// D [C] (all float32) and the slots' states [C, N] at the start of a slot.
+// D [C] (all float32) and the slots' states [C, N] at the start of a slot. max_q_len: the rows of the
+// step's longest sequence, or 0 when not known.
 extern "C" int ptl_selective_scan(void* out, int out_dtype, const float* xc, const float* z, long ldz,
                                   const float* r, long ldr, int b_off, int c_off, const float* w_dt,
                                   const float* dt_b, const float* A_log, const float* D, float* state,
                                   long slot_stride, const int32_t* q_start, const int32_t* state_slots,
-                                  int n_seqs, int C, int N, int R, hipStream_t st) {
+                                  int n_seqs, int max_q_len, int C, int N, int R, hipStream_t st) {
   if (n_seqs <= 0) return PTL_OK;
+  // a step of short sequences (decoded tokens) keeps fewer rows in LDS, so that more workgroups fit
+  const int chunk = max_q_len > 0 && max_q_len < SCHUNK ? max_q_len : SCHUNK;
   if (C <= 0 || N <= 0 || N > 256 || R <= 0 || n_seqs > 65535 ||
-      scan_lds_floats(N, R) * sizeof(float) > 150 * 1024)
+      scan_lds_floats(N, R, chunk) * sizeof(float) > 150 * 1024)
     return PTL_ERR_ARG;
   SelArgs a{out, xc, z, ldz, r, ldr, b_off, c_off, w_dt, dt_b, A_log, D, state, slot_stride, q_start,
-            state_slots, C, N, R};
+            state_slots, C, N, R, chunk};
   if (out_dtype == PTL_DTYPE_F32) return launch_scan<float>(a, n_seqs, st);
   if (out_dtype == PTL_DTYPE_BF16) return launch_scan<bf16_t>(a, n_seqs, st);
   return PTL_ERR_ARG;

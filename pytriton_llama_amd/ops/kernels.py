@@ -1833,6 +1833,6 @@ def selective_scan(xc: torch.Tensor, p: torch.Tensor, z_off: int, r: torch.Tenso
     _check(library.load("selective").ptl_selective_scan(
         _ptr(out), _dtype_code(out), _ptr(xc), _ptr(z), ctypes.c_long(p.stride(0)), _ptr(r),
         ctypes.c_long(r.stride(0)), int(b_off), int(c_off), _ptr(w_dt), _ptr(dt_bias), _ptr(A_log), _ptr(D),
-        _ptr(state), ctypes.c_long(state.stride(0)), _ptr(q_start), _ptr(state_slots), n, C, N, R, _stream()),
-        "selective_scan")
+        _ptr(state), ctypes.c_long(state.stride(0)), _ptr(q_start), _ptr(state_slots), n, int(max_q_len), C, N, R,
+        _stream()), "selective_scan")
     return out
