@@ -78,10 +78,15 @@ class PagedGroup:
     tables: Dict[Hashable, List[int]] = field(default_factory=dict)
 
     def first_needed_page(self, num_tokens: int) -> int:
-        """Index of the first page a query at position >= num_tokens can read."""
+        """Index of the first page inside the window of a query at position >= num_tokens."""
         if self.spec.window is None:
             return 0
         return max(0, num_tokens - self.spec.window + 1) // self.page_size
+
+    def kept_pages(self) -> int:
+        """Pages at the start of a sequence that are never given back: those of the first
+        positions that every later query reads."""
+        return -(-int(getattr(self.spec, "keep_first", 0)) // self.page_size)
 
 
 @dataclass
@@ -215,10 +220,11 @@ class CacheManager:
                 continue
             table = g.tables[req]
             first = min(g.first_needed_page(have), len(table))
-            dead = [table[i] for i in range(first) if table[i] >= 0]
+            behind = range(min(g.kept_pages(), first), first)
+            dead = [table[i] for i in behind if table[i] >= 0]
             if dead:
                 g.pool.give_back(dead)
-                for i in range(first):
+                for i in behind:
                     table[i] = RELEASED
                 n += len(dead)
         return n

@@ -2,6 +2,7 @@ from .model_config import ConfigError, LlamaConfig, RopeScaling, read_config_jso
 from .rubasun_config import RubasunConfig
 from .virusun_config import VirusunConfig
 from .matusun_config import MatusunConfig
+from .senavik_config import SenavikConfig
 from .engine_config import EngineConfig, parse_dtype
 from .registry import (MODEL_REGISTRY, Architecture, architecture_of, build_model,
                        config_from_dict, config_from_folder, register_model)

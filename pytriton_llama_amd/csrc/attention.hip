@@ -15,6 +15,12 @@
 // in page block_table[seq][p / page_size] at offset p % page_size.
 // window > 0 limits a query at position p to keys p-window+1 .. p; pages left
 // of every window may be gone (table entry < 0) and are never touched.
+// keep_first > 0 (with a window): the keys at positions below keep_first stay visible to every
+// later query, at their true positions; their pages are never given back. A kernel walks the
+// keys 0 .. min(keep_first, window start) - 1 and then the window, as one list ("walk index":
+// index v below n_kept is key v, index v from n_kept on is key v + shift).
+// sink (or null): one float a query head; the softmax denominator of that head holds exp(sink)
+// once more, a term without key and value that is not scaled.
 //
 // ptl_attention_generic: vector-FMA kernel, float32 math, storage type T
 // (float32 or bfloat16), any page size, any D up to 640 (beyond 256 with more LDS than a
@@ -38,7 +44,8 @@ attn_generic_kernel(TO* __restrict__ out, long out_stride, const T* __restrict__
                     const int32_t* __restrict__ q_start, const int32_t* __restrict__ ctx_len,
                     const int32_t* __restrict__ block_table, int bt_stride,
                     const int32_t* __restrict__ work_seq, const int32_t* __restrict__ work_qoff,
-                    int Hq, int Hkv, int maps, int Dk, int Dv, int page_size, int window, float scale) {
+                    int Hq, int Hkv, int maps, int Dk, int Dv, int page_size, int window, int keep_first,
+                    const float* __restrict__ sink, float scale) {
   extern __shared__ float lds[];
   float* Qs = lds;                   // [BM][Dk]
   float* Ks = Qs + BM * Dk;          // [BN][Dk+1]
@@ -71,7 +78,10 @@ attn_generic_kernel(TO* __restrict__ out, long out_stride, const T* __restrict__
   const int first_q = cached + qoff;
   const int k_end = min(ctx, first_q + rows);
   const int k_lo = window > 0 ? max(0, first_q - window + 1) : 0;
-  const int k_begin = (k_lo / BN) * BN;
+  // the walk: the kept first keys left of the window, then the keys from the window's start on
+  const int n_kept = min(max(keep_first, 0), k_lo);
+  const int shift = k_lo - n_kept;
+  const int n_walk = n_kept + (k_end - k_lo);
   const int nd = (Dv + 15) >> 4;
 
   float m_run = -INFINITY, l_run = 0.f;
@@ -79,13 +89,14 @@ attn_generic_kernel(TO* __restrict__ out, long out_stride, const T* __restrict__
 #pragma unroll
   for (int j = 0; j < NJ; ++j) acc[j] = 0.f;
 
-  for (int k0 = k_begin; k0 < k_end; k0 += BN) {
+  for (int k0 = 0; k0 < n_walk; k0 += BN) {
     __syncthreads();
     for (int i = tid; i < BN * Dk; i += 256) {
       const int n = i / Dk, d = i - n * Dk;
-      const int kp = k0 + n;
+      const int kw = k0 + n;
+      const int kp = kw < n_kept ? kw : kw + shift;
       float kv = 0.f;
-      if (kp >= k_lo && kp < k_end) {
+      if (kw < n_walk) {
         const int page = bt[kp / page_size];
         if (page >= 0)
           kv = to_float<T>(k_cache[(((size_t)page * Hk + kh) * page_size + (kp % page_size)) * Dk + d]);
@@ -94,9 +105,10 @@ attn_generic_kernel(TO* __restrict__ out, long out_stride, const T* __restrict__
     }
     for (int i = tid; i < BN * Dv; i += 256) {
       const int n = i / Dv, d = i - n * Dv;
-      const int kp = k0 + n;
+      const int kw = k0 + n;
+      const int kp = kw < n_kept ? kw : kw + shift;
       float vv = 0.f;
-      if (kp >= k_lo && kp < k_end) {
+      if (kw < n_walk) {
         const int page = bt[kp / page_size];
         if (page >= 0)
           vv = to_float<T>(v_cache[(((size_t)page * Hkv + vh) * page_size + (kp % page_size)) * Dv + d]);
@@ -110,12 +122,14 @@ attn_generic_kernel(TO* __restrict__ out, long out_stride, const T* __restrict__
 #pragma unroll
     for (int j = 0; j < BN / 16; ++j) {
       const int n = tc + 16 * j;
-      const int kp = k0 + n;
+      const int kw = k0 + n;
+      const int kp = kw < n_kept ? kw : kw + shift;
       const float* qr = Qs + tm * Dk;
       const float* kr = Ks + n * (Dk + 1);
       float dot = 0.f;
       for (int d = 0; d < Dk; ++d) dot = fmaf(qr[d], kr[d], dot);
-      const bool vis = row_valid && kp <= qpos && kp < ctx && (window <= 0 || kp > qpos - window);
+      const bool vis = row_valid && kw < n_walk && kp <= qpos &&
+                       (window <= 0 || kp > qpos - window || kp < keep_first);
       s[j] = vis ? dot * scale : -INFINITY;
       tmax = fmaxf(tmax, s[j]);
     }
@@ -139,7 +153,7 @@ attn_generic_kernel(TO* __restrict__ out, long out_stride, const T* __restrict__
     for (int j = 0; j < NJ; ++j) acc[j] *= alpha;
     __syncthreads();
 
-    const int n_lim = min(BN, k_end - k0);
+    const int n_lim = min(BN, n_walk - k0);
     for (int n = 0; n < n_lim; ++n) {
       const float p = Ss[tm * BN + n];
       const float* vr = Vs + n * Dv + tc;
@@ -150,7 +164,14 @@ attn_generic_kernel(TO* __restrict__ out, long out_stride, const T* __restrict__
   }
 
   if (row_valid) {
-    const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
+    float den = l_run, f = 1.f;
+    if (sink) {                            // one more term of the denominator: exp(sink)
+      const float sk = sink[head];
+      const float mx = fmaxf(m_run, sk);
+      f = expf(m_run - mx);
+      den = l_run * f + expf(sk - mx);
+    }
+    const float inv = den > 0.f ? f / den : 0.f;
     TO* o = out + (size_t)(qs + qoff + tm) * out_stride + head * Dv + tc;
 #pragma unroll
     for (int j = 0; j < NJ; ++j)
@@ -164,7 +185,7 @@ static int launch_generic(void* out, long out_stride, const void* q, long q_stri
                           const int32_t* ctx_len, const int32_t* block_table, int bt_stride,
                           const int32_t* work_seq, const int32_t* work_qoff, int n_work,
                           int Hq, int Hkv, int maps, int Dk, int Dv, int page_size, int window,
-                          float scale, hipStream_t stream) {
+                          int keep_first, const float* sink, float scale, hipStream_t stream) {
   const size_t lds = (size_t)(BM * Dk + BN * (Dk + 1) + BN * Dv + BM * BN) * sizeof(float);
   if (lds > 64 * 1024) {
     // more dynamic LDS than a kernel may ask for without saying so beforehand (wide heads only)
@@ -182,7 +203,7 @@ static int launch_generic(void* out, long out_stride, const void* q, long q_stri
   attn_generic_kernel<T, TO, BN, NJ><<<grid, 256, lds, stream>>>(
       (TO*)out, out_stride, (const T*)q, q_stride, (const T*)k_cache, (const T*)v_cache, q_start,
       ctx_len, block_table, bt_stride, work_seq, work_qoff, Hq, Hkv, maps, Dk, Dv, page_size, window,
-      scale);
+      keep_first, sink, scale);
   return ptl_launch_status();
 }
 
@@ -196,7 +217,8 @@ extern "C" int ptl_attention_generic_kv(void* out, long out_stride, int out_f32,
                                         const int32_t* block_table, int bt_stride,
                                         const int32_t* work_seq, const int32_t* work_qoff, int n_work,
                                         int Hq, int Hkv, int maps, int Dk, int Dv, int page_size,
-                                        int window, float scale, int dtype, hipStream_t stream) {
+                                        int window, int keep_first, const float* sink, float scale,
+                                        int dtype, hipStream_t stream) {
   if (n_work <= 0) return PTL_OK;
   if (Hq <= 0 || Hkv <= 0 || maps <= 0 || Hq % maps || (Hq / maps) % Hkv || Dk <= 0 || Dv <= 0 ||
       Dk > 640 || Dv > 640 || page_size <= 0 || Hq > 65535)
@@ -204,7 +226,7 @@ extern "C" int ptl_attention_generic_kv(void* out, long out_stride, int out_f32,
 #define GO(T, TO, BN, NJ)                                                                         \
   launch_generic<T, TO, BN, NJ>(out, out_stride, q, q_stride, k_cache, v_cache, q_start, ctx_len, \
                                 block_table, bt_stride, work_seq, work_qoff, n_work, Hq, Hkv,    \
-                                maps, Dk, Dv, page_size, window, scale, stream)
+                                maps, Dk, Dv, page_size, window, keep_first, sink, scale, stream)
 #define GO_SIZES(T, TO)                                                                           \
   {                                                                                               \
     /* wide heads (a latent cache of 512 + 64, say): 40 columns a thread, 16 keys a turn */       \
@@ -227,11 +249,12 @@ extern "C" int ptl_attention_generic(void* out, long out_stride, const void* q, 
                                      const int32_t* q_start, const int32_t* ctx_len,
                                      const int32_t* block_table, int bt_stride,
                                      const int32_t* work_seq, const int32_t* work_qoff, int n_work,
-                                     int Hq, int Hkv, int D, int page_size, int window, float scale,
+                                     int Hq, int Hkv, int D, int page_size, int window,
+                                     int keep_first, const float* sink, float scale,
                                      int dtype, hipStream_t stream) {
   return ptl_attention_generic_kv(out, out_stride, 0, q, q_stride, k_cache, v_cache, q_start, ctx_len,
                                   block_table, bt_stride, work_seq, work_qoff, n_work, Hq, Hkv, 1, D,
-                                  D, page_size, window, scale, dtype, stream);
+                                  D, page_size, window, keep_first, sink, scale, dtype, stream);
 }
 
 // ===========================================================================
@@ -292,8 +315,8 @@ attn_decode_kernel(TO* __restrict__ out, long out_stride, const T* __restrict__ 
                    const int32_t* __restrict__ q_start, const int32_t* __restrict__ ctx_len,
                    const int32_t* __restrict__ block_table, int bt_stride,
                    float* __restrict__ part_acc, float* __restrict__ part_ml,
-                   int Hq, int Hkv, int maps, int Dk, int Dv, int page_size, int window, float scale,
-                   int num_splits, int groups_per_kv) {
+                   int Hq, int Hkv, int maps, int Dk, int Dv, int page_size, int window, int keep_first,
+                   const float* __restrict__ sink, float scale, int num_splits, int groups_per_kv) {
   constexpr int KPW = 64 / LPK;           // keys a wave reads per turn
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int seq = blockIdx.x;
@@ -308,11 +331,14 @@ attn_decode_kernel(TO* __restrict__ out, long out_stride, const T* __restrict__ 
   const int row = q_start[seq];
   const int ctx = ctx_len[seq];
   const int k_lo = window > 0 ? max(0, ctx - window) : 0;
-  const int span = ctx - k_lo;
+  // the walk: the kept first keys left of the window, then the window (indices, not positions)
+  const int n_kept = min(max(keep_first, 0), k_lo);
+  const int shift = k_lo - n_kept;
+  const int span = ctx - shift;
   const int tile = 4 * KPW;
   const int per_split = ((span + num_splits - 1) / num_splits + tile - 1) / tile * tile;
-  const int k_begin = k_lo + split * per_split;
-  const int k_end = min(ctx, k_begin + per_split);
+  const int k_begin = split * per_split;
+  const int k_end = min(span, k_begin + per_split);
   const int32_t* bt = block_table + (size_t)seq * bt_stride;
 
   const int c = lane % LPK;                 // which 16 elements of the head this lane owns
@@ -340,8 +366,9 @@ attn_decode_kernel(TO* __restrict__ out, long out_stride, const T* __restrict__ 
   }
 
   for (int kb = k_begin + wave * KPW; kb < k_end; kb += tile) {
-    const int kp = kb + ks;
-    const bool valid = kp < k_end;
+    const int kw = kb + ks;
+    const bool valid = kw < k_end;
+    const int kp = kw < n_kept ? kw : kw + shift;
     float kf[DEC_CHUNK], vf[DEC_CHUNK];
 #pragma unroll
     for (int j = 0; j < DEC_CHUNK; ++j) { kf[j] = 0.f; vf[j] = 0.f; }
@@ -424,6 +451,13 @@ attn_decode_kernel(TO* __restrict__ out, long out_stride, const T* __restrict__ 
     }
     const int head = (head0 + h) * maps + map;
     if (num_splits == 1) {
+      if (sink) {                          // one more term of the denominator: exp(sink)
+        const float sk = sink[head];
+        const float mx = fmaxf(mn, sk);
+        const float f = expf(mn - mx);
+        ll = ll * f + expf(sk - mx);
+        a *= f;
+      }
       out[(size_t)row * out_stride + (size_t)head * Dv + d] = from_float<TO>(ll > 0.f ? a / ll : 0.f);
     } else {
       const size_t pi = ((size_t)seq * Hq + head) * num_splits + split;
@@ -437,7 +471,7 @@ template <typename T>
 __global__ void __launch_bounds__(64)
 attn_decode_merge_kernel(T* __restrict__ out, long out_stride, const int32_t* __restrict__ q_start,
                          const float* __restrict__ part_acc, const float* __restrict__ part_ml,
-                         int Hq, int D, int num_splits) {
+                         int Hq, int D, int num_splits, const float* __restrict__ sink) {
   // one wave per (sequence, head): lanes take the splits' (max, denominator) side by side,
   // then the head dimension, with the splits' weights in LDS. The partial results come from
   // other compute units' writes, a long way off: the first 16 splits of the lane's first
@@ -455,6 +489,8 @@ attn_decode_merge_kernel(T* __restrict__ out, long out_stride, const int32_t* __
   float mn = -INFINITY;
   for (int s = lane; s < num_splits; s += 64) mn = fmaxf(mn, part_ml[(base + s) * 2]);
   mn = wave_max(mn);
+  const float sk = sink ? sink[head] : -INFINITY;      // the denominator's term without a key
+  mn = fmaxf(mn, sk);
   const float ms = mn == -INFINITY ? 0.f : mn;
   float ll = 0.f;
   for (int s = lane; s < num_splits; s += 64) {
@@ -463,6 +499,7 @@ attn_decode_merge_kernel(T* __restrict__ out, long out_stride, const int32_t* __
     ll += part_ml[(base + s) * 2 + 1] * w;
   }
   ll = wave_sum(ll);
+  if (sink) ll += expf(sk - ms);
   __syncthreads();
   const float inv = ll > 0.f ? 1.0f / ll : 0.f;
   for (int d = lane; d < D; d += 64) {
@@ -485,8 +522,8 @@ static int launch_decode(void* out, long out_stride, const void* q, long q_strid
                          const void* k_cache, const void* v_cache, const int32_t* q_start,
                          const int32_t* ctx_len, const int32_t* block_table, int bt_stride,
                          float* part_acc, float* part_ml, int n_seq, int Hq, int Hkv, int maps, int Dk,
-                         int Dv, int page_size, int window, float scale, int num_splits,
-                         hipStream_t stream) {
+                         int Dv, int page_size, int window, int keep_first, const float* sink,
+                         float scale, int num_splits, hipStream_t stream) {
   constexpr int GT = 4;
   const int G = (Hq / maps) / Hkv;
   const int groups = (G + GT - 1) / GT;
@@ -495,12 +532,12 @@ static int launch_decode(void* out, long out_stride, const void* q, long q_strid
   attn_decode_kernel<T, TO, GT, LPK><<<grid, 256, lds, stream>>>(
       (TO*)out, out_stride, (const T*)q, q_stride, (const T*)k_cache, (const T*)v_cache, q_start,
       ctx_len, block_table, bt_stride, part_acc, part_ml, Hq, Hkv, maps, Dk, Dv, page_size, window,
-      scale, num_splits, groups);
+      keep_first, sink, scale, num_splits, groups);
   if (hipGetLastError() != hipSuccess) return PTL_ERR_LAUNCH;
   if (num_splits > 1) {
     dim3 mgrid(n_seq, Hq);
     attn_decode_merge_kernel<TO><<<mgrid, 64, 0, stream>>>((TO*)out, out_stride, q_start, part_acc,
-                                                          part_ml, Hq, Dv, num_splits);
+                                                          part_ml, Hq, Dv, num_splits, sink);
   }
   return ptl_launch_status();
 }
@@ -515,7 +552,8 @@ extern "C" int ptl_attention_decode_kv(void* out, long out_stride, int out_f32, 
                                        const int32_t* q_start, const int32_t* ctx_len,
                                        const int32_t* block_table, int bt_stride, float* part_acc,
                                        float* part_ml, int n_seq, int Hq, int Hkv, int maps, int Dk,
-                                       int Dv, int page_size, int window, float scale, int num_splits,
+                                       int Dv, int page_size, int window, int keep_first,
+                                       const float* sink, float scale, int num_splits,
                                        int dtype, hipStream_t stream) {
   if (n_seq <= 0) return PTL_OK;
   if (Hq <= 0 || Hkv <= 0 || maps <= 0 || Hq % maps || (Hq / maps) % Hkv || Dk <= 0 || Dk % 16 ||
@@ -527,8 +565,8 @@ extern "C" int ptl_attention_decode_kv(void* out, long out_stride, int out_f32, 
   while (lpk < chunks) lpk <<= 1;
 #define GO(T, TO, L) launch_decode<T, TO, L>(out, out_stride, q, q_stride, k_cache, v_cache, q_start, \
                                              ctx_len, block_table, bt_stride, part_acc, part_ml,    \
-                                             n_seq, Hq, Hkv, maps, Dk, Dv, page_size, window, scale, \
-                                             num_splits, stream)
+                                             n_seq, Hq, Hkv, maps, Dk, Dv, page_size, window,       \
+                                             keep_first, sink, scale, num_splits, stream)
 #define BY_LPK(T, TO)                                                                              \
   switch (lpk) {                                                                                   \
     case 1: return GO(T, TO, 1);                                                                   \
@@ -553,11 +591,11 @@ extern "C" int ptl_attention_decode(void* out, long out_stride, const void* q, l
                                     const int32_t* q_start, const int32_t* ctx_len,
                                     const int32_t* block_table, int bt_stride, float* part_acc,
                                     float* part_ml, int n_seq, int Hq, int Hkv, int D, int page_size,
-                                    int window, float scale, int num_splits, int dtype,
-                                    hipStream_t stream) {
+                                    int window, int keep_first, const float* sink, float scale,
+                                    int num_splits, int dtype, hipStream_t stream) {
   return ptl_attention_decode_kv(out, out_stride, 0, q, q_stride, k_cache, v_cache, q_start, ctx_len,
                                  block_table, bt_stride, part_acc, part_ml, n_seq, Hq, Hkv, 1, D, D,
-                                 page_size, window, scale, num_splits, dtype, stream);
+                                 page_size, window, keep_first, sink, scale, num_splits, dtype, stream);
 }
 
 // ===========================================================================
@@ -598,8 +636,8 @@ attn_decode_mfma_kernel(bf16_t* __restrict__ out, long out_stride, const bf16_t*
                         const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ q_start,
                         const int32_t* __restrict__ ctx_len, const int32_t* __restrict__ block_table,
                         int bt_stride, float* __restrict__ part_acc, float* __restrict__ part_ml,
-                        int Hq, int Hkv, int page_size, int page_shift, int window, float scale_log2,
-                        int num_splits) {
+                        int Hq, int Hkv, int page_size, int page_shift, int window, int keep_first,
+                        const float* __restrict__ sink, float scale_log2, int num_splits) {
   constexpr int D = 32 * NDT;
   constexpr int NT = 2 * NDT;             // 16-wide tiles of the head dimension
   constexpr int TILE = 64 * UNR;          // keys per turn of the workgroup
@@ -614,11 +652,16 @@ attn_decode_mfma_kernel(bf16_t* __restrict__ out, long out_stride, const bf16_t*
   const int row = q_start[seq];
   const int ctx = ctx_len[seq];
   const int k_lo = window > 0 ? max(0, ctx - window) : 0;
-  const int span = ctx - k_lo;
+  // the walk: the kept first keys left of the window, then the window; k_begin, k_end and the
+  // keys of a turn are indices of the walk, key_at gives the position
+  const int n_kept = min(max(keep_first, 0), k_lo);
+  const int shift = k_lo - n_kept;
+  const int span = ctx - shift;
   const int per_split = ((span + num_splits - 1) / num_splits + TILE - 1) / TILE * TILE;
-  const int k_begin = k_lo + split * per_split;
-  const int k_end = min(ctx, k_begin + per_split);
+  const int k_begin = split * per_split;
+  const int k_end = min(span, k_begin + per_split);
   const int turns = (k_end - k_begin + TILE - 1) / TILE;
+  auto key_at = [&](int kw) { return kw < n_kept ? kw : kw + shift; };
   const int32_t* bt = block_table + (size_t)seq * bt_stride;
   const uint32_t page_bytes = (uint32_t)Hkv * page_size * D * 2;
   const int page_mask = page_size - 1;
@@ -657,11 +700,11 @@ attn_decode_mfma_kernel(bf16_t* __restrict__ out, long out_stride, const bf16_t*
 #pragma unroll
     for (int u = 0; u < UNR; ++u) {
       const int kp = kc + 16 * u + ln;
-      pk[u] = (turn < turns && kp < k_end) ? bt[kp >> page_shift] : -1;
+      pk[u] = (turn < turns && kp < k_end) ? bt[key_at(kp) >> page_shift] : -1;
 #pragma unroll
       for (int i = 0; i < VCH; ++i) {
         const int vp = kc + 16 * u + vrow[i];
-        pv[u][i] = (turn < turns && vp < k_end) ? bt[vp >> page_shift] : -1;
+        pv[u][i] = (turn < turns && vp < k_end) ? bt[key_at(vp) >> page_shift] : -1;
       }
     }
   };
@@ -669,7 +712,7 @@ attn_decode_mfma_kernel(bf16_t* __restrict__ out, long out_stride, const bf16_t*
     const int kc = first_key(turn);
 #pragma unroll
     for (int u = 0; u < UNR; ++u) {
-      const int kp = kc + 16 * u + ln;
+      const int kp = key_at(kc + 16 * u + ln);
       const char* kr = k_head + (size_t)(uint32_t)max(pk[u], 0) * page_bytes +
                        (uint32_t)(((kp & page_mask) * D + 8 * lg) * 2);
 #pragma unroll
@@ -677,7 +720,7 @@ attn_decode_mfma_kernel(bf16_t* __restrict__ out, long out_stride, const bf16_t*
         kf[u][kk].u = pk[u] >= 0 ? load_once(kr + 64 * kk) : make_uint4(0, 0, 0, 0);
 #pragma unroll
       for (int i = 0; i < VCH; ++i) {
-        const int vp = kc + 16 * u + vrow[i];
+        const int vp = key_at(kc + 16 * u + vrow[i]);
         vg[u][i] = make_uint4(0, 0, 0, 0);              // rows past the end read as zeros
         if (pv[u][i] >= 0)
           vg[u][i] = load_once(v_head + (size_t)(uint32_t)pv[u][i] * page_bytes +
@@ -788,6 +831,13 @@ attn_decode_mfma_kernel(bf16_t* __restrict__ out, long out_stride, const bf16_t*
     }
     const int head = head0 + h;
     if (num_splits == 1) {
+      if (sink) {                          // one more term of the denominator: exp(sink)
+        const float sk = sink[head] * 1.4426950408889634f;
+        const float mx = fmaxf(mn, sk);
+        const float f = __builtin_amdgcn_exp2f(mn - mx);
+        ll = ll * f + __builtin_amdgcn_exp2f(sk - mx);
+        a *= f;
+      }
       out[(size_t)row * out_stride + (size_t)head * D + d] = float_to_bf16(ll > 0.f ? a / ll : 0.f);
     } else {
       const size_t pi = ((size_t)seq * Hq + head) * num_splits + split;
@@ -803,8 +853,8 @@ static int launch_decode_mfma(void* out, long out_stride, const void* q, long q_
                               const void* k_cache, const void* v_cache, const int32_t* q_start,
                               const int32_t* ctx_len, const int32_t* block_table, int bt_stride,
                               float* part_acc, float* part_ml, int n_seq, int Hq, int Hkv,
-                              int page_size, int window, float scale, int num_splits,
-                              hipStream_t stream) {
+                              int page_size, int window, int keep_first, const float* sink,
+                              float scale, int num_splits, hipStream_t stream) {
   constexpr int D = 32 * NDT;
   dim3 grid(n_seq, Hkv, num_splits);
   int page_shift = 0;
@@ -815,12 +865,12 @@ static int launch_decode_mfma(void* out, long out_stride, const void* q, long q_
   attn_decode_mfma_kernel<NDT, UNR><<<grid, 256, lds, stream>>>(
       (bf16_t*)out, out_stride, (const bf16_t*)q, q_stride, (const bf16_t*)k_cache,
       (const bf16_t*)v_cache, q_start, ctx_len, block_table, bt_stride, part_acc, part_ml, Hq, Hkv,
-      page_size, page_shift, window, scale * 1.4426950408889634f, num_splits);
+      page_size, page_shift, window, keep_first, sink, scale * 1.4426950408889634f, num_splits);
   if (hipGetLastError() != hipSuccess) return PTL_ERR_LAUNCH;
   if (num_splits > 1) {
     dim3 mgrid(n_seq, Hq);
     attn_decode_merge_kernel<bf16_t><<<mgrid, 64, 0, stream>>>((bf16_t*)out, out_stride, q_start,
-                                                              part_acc, part_ml, Hq, D, num_splits);
+                                                              part_acc, part_ml, Hq, D, num_splits, sink);
   }
   return ptl_launch_status();
 }
@@ -831,8 +881,8 @@ extern "C" int ptl_attention_decode_mfma(void* out, long out_stride, const void*
                                          const int32_t* q_start, const int32_t* ctx_len,
                                          const int32_t* block_table, int bt_stride, float* part_acc,
                                          float* part_ml, int n_seq, int Hq, int Hkv, int D,
-                                         int page_size, int window, float scale, int num_splits,
-                                         int unroll, hipStream_t stream) {
+                                         int page_size, int window, int keep_first, const float* sink,
+                                         float scale, int num_splits, int unroll, hipStream_t stream) {
   if (n_seq <= 0) return PTL_OK;
   if (Hq <= 0 || Hkv <= 0 || Hq % Hkv || Hq / Hkv > 16 || D <= 0 || D % 32 || D > 128 ||
       page_size <= 0 || (page_size & (page_size - 1)) ||
@@ -842,7 +892,8 @@ extern "C" int ptl_attention_decode_mfma(void* out, long out_stride, const void*
   if (unroll == 0) unroll = 2;
 #define GO(N, U) launch_decode_mfma<N, U>(out, out_stride, q, q_stride, k_cache, v_cache, q_start,    \
                                           ctx_len, block_table, bt_stride, part_acc, part_ml, n_seq, \
-                                          Hq, Hkv, page_size, window, scale, num_splits, stream)
+                                          Hq, Hkv, page_size, window, keep_first, sink, scale,       \
+                                          num_splits, stream)
   if (unroll == 1) {
     switch (D / 32) {
       case 1: return GO(1, 1);

@@ -74,7 +74,8 @@ attn_prefill_mfma_kernel(TO* __restrict__ out, long out_stride, const bf16_t* __
                          const int32_t* __restrict__ ctx_len, const int32_t* __restrict__ block_table,
                          int bt_stride, const int32_t* __restrict__ work_seq,
                          const int32_t* __restrict__ work_qoff, int n_work, int Hq, int Hkv, int maps,
-                         int page_size, int page_shift, int window, float scale_log2) {
+                         int page_size, int page_shift, int window, int keep_first,
+                         const float* __restrict__ sink, float scale_log2) {
   constexpr int DK = 32 * NDK, DV = 32 * NDV;
   constexpr int PBM = 64 * RT;
   constexpr int CPRK = DK / 8, CPRV = DV / 8;      // 16-byte chunks per row
@@ -156,10 +157,15 @@ attn_prefill_mfma_kernel(TO* __restrict__ out, long out_stride, const bf16_t* __
   // and bfloat16 probabilities hold as well as values below 1, and nothing is rescaled
   const float lazy = 8.0f / scale_log2;
 
-  const int k_end = min(ctx, first_q + rows);
+  // The keys this block walks, as one list: the kept first keys left of the window (positions
+  // 0 .. n_kept - 1), then the positions from the window's start on. Tiles, k0 and the rows of a
+  // tile are indices of that list; key_at gives the position (the identity without a window).
   const int k_lo = window > 0 ? max(0, first_q - window + 1) : 0;
-  const int k_begin = (k_lo / PF_BN) * PF_BN;
-  const int n_tiles = (k_end - k_begin + PF_BN - 1) / PF_BN;
+  const int n_kept = min(max(keep_first, 0), k_lo);
+  const int shift = k_lo - n_kept;
+  const int k_end = min(ctx, first_q + rows) - shift;
+  const int n_tiles = (k_end + PF_BN - 1) / PF_BN;
+  auto key_at = [&](int kw) { return kw < n_kept ? kw : kw + shift; };
 
   // This thread's chunks of a tile. A wave's load instruction fills 64 consecutive 16-byte
   // slots of LDS, lane l the l-th; slot s holds row s / CPR, chunk (s % CPR) ^ swz(row).
@@ -186,28 +192,28 @@ attn_prefill_mfma_kernel(TO* __restrict__ out, long out_stride, const bf16_t* __
   const int page_mask = page_size - 1;                                // page sizes are powers of two
   // a tile that lies wholly inside the keys this block sees needs no tests (uniform)
   auto whole = [&](int t) {
-    const int k0 = k_begin + t * PF_BN;
-    return t < n_tiles && k0 >= k_lo && k0 + PF_BN <= k_end;
+    const int k0 = t * PF_BN;
+    return t < n_tiles && k0 + PF_BN <= k_end;
   };
   auto load_pages = [&](int t) {
-    const int k0 = k_begin + t * PF_BN;
+    const int k0 = t * PF_BN;
     if (whole(t)) {
 #pragma unroll
-      for (int i = 0; i < NCHK; ++i) pgk[i] = bt[(k0 + crowk[i]) >> page_shift];
+      for (int i = 0; i < NCHK; ++i) pgk[i] = bt[key_at(k0 + crowk[i]) >> page_shift];
 #pragma unroll
-      for (int i = 0; i < NCHV; ++i) pgv[i] = bt[(k0 + crowv[i]) >> page_shift];
+      for (int i = 0; i < NCHV; ++i) pgv[i] = bt[key_at(k0 + crowv[i]) >> page_shift];
     } else {
 #pragma unroll
       for (int i = 0; i < NCHK; ++i) {
         const int kp = k0 + crowk[i];
         pgk[i] = -1;
-        if (t < n_tiles && kp >= k_lo && kp < k_end) pgk[i] = bt[kp >> page_shift];
+        if (t < n_tiles && kp < k_end) pgk[i] = bt[key_at(kp) >> page_shift];
       }
 #pragma unroll
       for (int i = 0; i < NCHV; ++i) {
         const int kp = k0 + crowv[i];
         pgv[i] = -1;
-        if (t < n_tiles && kp >= k_lo && kp < k_end) pgv[i] = bt[kp >> page_shift];
+        if (t < n_tiles && kp < k_end) pgv[i] = bt[key_at(kp) >> page_shift];
       }
     }
   };
@@ -219,12 +225,12 @@ attn_prefill_mfma_kernel(TO* __restrict__ out, long out_stride, const bf16_t* __
         (__attribute__((address_space(3))) void*)(tile_lds + 512 * chunk), 16, 0, 0);
   };
   auto fetch = [&](int t, bf16_t* Kb, bf16_t* Vb) {
-    const int k0 = k_begin + t * PF_BN;
+    const int k0 = t * PF_BN;
     const bool all = whole(t);
 #pragma unroll
     for (int i = 0; i < NCHK; ++i) {
       if (all || pgk[i] >= 0) {
-        const uint32_t in_page = (uint32_t)(((k0 + crowk[i]) & page_mask) * DK + ccolk[i]) * 2;
+        const uint32_t in_page = (uint32_t)((key_at(k0 + crowk[i]) & page_mask) * DK + ccolk[i]) * 2;
         to_lds(k_head, (uint64_t)(uint32_t)pgk[i] * page_bytes_k + in_page, Kb, wave_u * NCHK + i);
       } else {                                    // rows outside the keys read as zeros
         *reinterpret_cast<uint4*>(Kb + 8 * (64 * (wave_u * NCHK + i) + lane)) = make_uint4(0, 0, 0, 0);
@@ -233,7 +239,7 @@ attn_prefill_mfma_kernel(TO* __restrict__ out, long out_stride, const bf16_t* __
 #pragma unroll
     for (int i = 0; i < NCHV; ++i) {
       if (all || pgv[i] >= 0) {
-        const uint32_t in_page = (uint32_t)(((k0 + crowv[i]) & page_mask) * DV + ccolv[i]) * 2;
+        const uint32_t in_page = (uint32_t)((key_at(k0 + crowv[i]) & page_mask) * DV + ccolv[i]) * 2;
         to_lds(v_head, (uint64_t)(uint32_t)pgv[i] * page_bytes_v + in_page, Vb, wave_u * NCHV + i);
       } else {
         *reinterpret_cast<uint4*>(Vb + 8 * (64 * (wave_u * NCHV + i) + lane)) = make_uint4(0, 0, 0, 0);
@@ -280,8 +286,10 @@ attn_prefill_mfma_kernel(TO* __restrict__ out, long out_stride, const bf16_t* __
         for (int kt = 0; kt < 4; ++kt)
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
-            const int key = k0 + 16 * kt + 4 * lg + i;
-            const bool vis = key <= qpos[r] && key < k_end && (window <= 0 || key > qpos[r] - window);
+            const int kw = k0 + 16 * kt + 4 * lg + i;
+            const int key = key_at(kw);
+            const bool vis = key <= qpos[r] && kw < k_end &&
+                             (window <= 0 || key > qpos[r] - window || key < keep_first);
             st[r][kt][i] = vis ? st[r][kt][i] : -INFINITY;
           }
       }
@@ -340,13 +348,14 @@ attn_prefill_mfma_kernel(TO* __restrict__ out, long out_stride, const bf16_t* __
   // one turn: tile t + 1 sets out for the other buffer (everyone left it before the last
   // barrier), tile t is used, and what was loaded is waited for before the barrier
   auto turn = [&](int t, bf16_t* Kb, bf16_t* Vb, bf16_t* Kn, bf16_t* Vn) {
-    const int k0 = k_begin + t * PF_BN;
+    const int k0 = t * PF_BN;
     if (t + 1 < n_tiles) {
       fetch(t + 1, Kn, Vn);
       load_pages(t + 2);
     }
     // a wave whose rows all lie before this tile has nothing to do in it
-    if (wave_has_rows && k0 <= wave_max_q) {
+    if (wave_has_rows && key_at(k0) <= wave_max_q) {
+      // (without a window an index of the walk is a position)
       const bool need_mask = (k0 + PF_BN - 1 > wave_min_q) || (k0 + PF_BN > k_end) || window > 0;
       if (need_mask)
         tile(k0, Kb, Vb, std::true_type{});
@@ -368,7 +377,9 @@ attn_prefill_mfma_kernel(TO* __restrict__ out, long out_stride, const bf16_t* __
 
 #pragma unroll
   for (int r = 0; r < RT; ++r) {
-    const float l = o[r][2 * NDV][0];          // every row of that tile holds the column's sum
+    float l = o[r][2 * NDV][0];                // every row of that tile holds the column's sum
+    // one more term of the denominator: exp(sink), in the units of what was summed
+    if (sink) l += __builtin_amdgcn_exp2f(sink[head] * 1.4426950408889634f - m_run[r] * scale_log2);
     if (row_ok[r]) {
       const float inv = l > 0.f ? 1.0f / l : 0.f;
       const int my_row = 16 * (RT * wave + r) + ln;
@@ -391,7 +402,7 @@ static int launch_prefill_mfma(void* out, long out_stride, const void* q, long q
                                const int32_t* ctx_len, const int32_t* block_table, int bt_stride,
                                const int32_t* work_seq, const int32_t* work_qoff, int n_work,
                                int n_groups, int Hq, int Hkv, int maps, int page_size, int window,
-                               float scale, hipStream_t stream) {
+                               int keep_first, const float* sink, float scale, hipStream_t stream) {
   dim3 grid(Hq, n_groups < 65535 ? n_groups : 65535);
   int page_shift = -1;
   for (int sh = 0; sh < 31; ++sh)
@@ -399,7 +410,8 @@ static int launch_prefill_mfma(void* out, long out_stride, const void* q, long q
   attn_prefill_mfma_kernel<NDK, NDV, RT, TO><<<grid, 256, 0, stream>>>(
       (TO*)out, out_stride, (const bf16_t*)q, q_stride, (const bf16_t*)k_cache,
       (const bf16_t*)v_cache, q_start, ctx_len, block_table, bt_stride, work_seq, work_qoff,
-      n_work, Hq, Hkv, maps, page_size, page_shift, window, scale * 1.4426950408889634f);
+      n_work, Hq, Hkv, maps, page_size, page_shift, window, keep_first, sink,
+      scale * 1.4426950408889634f);
   return ptl_launch_status();
 }
 
@@ -410,10 +422,12 @@ static int prefill_same_size(int nd, void* out, long out_stride, const void* q, 
                              const void* k_cache, const void* v_cache, const int32_t* q_start,
                              const int32_t* ctx_len, const int32_t* block_table, int bt_stride,
                              const int32_t* work_seq, const int32_t* work_qoff, int n_work, int n_groups,
-                             int Hq, int Hkv, int page_size, int window, float scale, hipStream_t stream) {
+                             int Hq, int Hkv, int page_size, int window, int keep_first, const float* sink,
+                             float scale, hipStream_t stream) {
 #define GO(N) launch_prefill_mfma<N, N, RT, bf16_t>(out, out_stride, q, q_stride, k_cache, v_cache, q_start, \
                                                     ctx_len, block_table, bt_stride, work_seq, work_qoff,  \
-                                                    n_work, n_groups, Hq, Hkv, 1, page_size, window, scale, stream)
+                                                    n_work, n_groups, Hq, Hkv, 1, page_size, window,     \
+                                                    keep_first, sink, scale, stream)
   switch (nd) {
     case 1: return GO(1);
     case 2: return GO(2);
@@ -434,8 +448,8 @@ extern "C" int ptl_attention_prefill_mfma(void* out, long out_stride, const void
                                           const int32_t* work_seq, const int32_t* work_qoff,
                                           int n_work, int n_groups, int block_rows, int Hq,
                                           int Hkv, int D,
-                                          int page_size, int window, float scale,
-                                          hipStream_t stream) {
+                                          int page_size, int window, int keep_first,
+                                          const float* sink, float scale, hipStream_t stream) {
   if (n_work <= 0) return PTL_OK;
   if (Hq <= 0 || Hkv <= 0 || Hq % Hkv || D % 32 || D <= 0 || D > 128 || page_size <= 0 ||
       (page_size & (page_size - 1)) || (long)Hkv * page_size * D * 2 >= (1L << 32) ||
@@ -445,10 +459,10 @@ extern "C" int ptl_attention_prefill_mfma(void* out, long out_stride, const void
   if (block_rows == 64)
     return prefill_same_size<1>(D / 32, out, out_stride, q, q_stride, k_cache, v_cache, q_start, ctx_len,
                                 block_table, bt_stride, work_seq, work_qoff, n_work, n_groups, Hq, Hkv,
-                                page_size, window, scale, stream);
+                                page_size, window, keep_first, sink, scale, stream);
   return prefill_same_size<2>(D / 32, out, out_stride, q, q_stride, k_cache, v_cache, q_start, ctx_len,
                               block_table, bt_stride, work_seq, work_qoff, n_work, n_groups, Hq, Hkv,
-                              page_size, window, scale, stream);
+                              page_size, window, keep_first, sink, scale, stream);
 }
 
 // The general form: q [T, Hq, Dk] with Hq = heads * maps, k_cache [pages, Hkv * maps, page_size,
@@ -460,8 +474,8 @@ extern "C" int ptl_attention_prefill_mfma_kv(void* out, long out_stride, int out
                                              const int32_t* block_table, int bt_stride,
                                              const int32_t* work_seq, const int32_t* work_qoff,
                                              int n_work, int n_groups, int Hq, int Hkv, int maps, int Dk,
-                                             int Dv, int page_size, int window, float scale,
-                                             hipStream_t stream) {
+                                             int Dv, int page_size, int window, int keep_first,
+                                             const float* sink, float scale, hipStream_t stream) {
   if (n_work <= 0) return PTL_OK;
   if (Hq <= 0 || Hkv <= 0 || maps <= 0 || Hq % maps || (Hq / maps) % Hkv || Dk % 32 || Dk <= 0 ||
       Dk > 128 || Dv % 32 || Dv <= 0 || Dv > 128 || page_size <= 0 || (page_size & (page_size - 1)) ||
@@ -471,7 +485,7 @@ extern "C" int ptl_attention_prefill_mfma_kv(void* out, long out_stride, int out
 #define GO(NK, NV, TO)                                                                                  \
   launch_prefill_mfma<NK, NV, 1, TO>(out, out_stride, q, q_stride, k_cache, v_cache, q_start, ctx_len, \
                                      block_table, bt_stride, work_seq, work_qoff, n_work, n_groups, Hq, \
-                                     Hkv, maps, page_size, window, scale, stream)
+                                     Hkv, maps, page_size, window, keep_first, sink, scale, stream)
 #define BY_V(NK, TO)                   \
   switch (Dv / 32) {                   \
     case 1: return GO(NK, 1, TO);      \

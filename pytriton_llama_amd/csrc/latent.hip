@@ -6,12 +6,13 @@
 //   score_h(i, j) = qn_h(i) . (Uk_h c_j) + qr_h(i) . kr_j = (Uk_h^T qn_h(i)) . c_j + qr_h(i) . kr_j
 //   out_h(i)      = Uv_h sum_j p_h(i, j) c_j
 //
-// ptl_latent_prepare: per token, from the row of projections [q | down-projection]: the RMS
-//   norm of the first R entries of the down-projection (float32, weight w), the rotation of its
-//   last dr entries, both written to the cache slot [c | kr]; and the rotation of the dr
-//   rotated entries of every query head, written behind the R entries that
-//   ptl_gemm_heads_nt fills (query rows [H, R + dr]). Rotation: neighbouring pairs (2i, 2i+1)
-//   of the first 2 * n_pairs entries, angle = position * inv_freq[i], float32; the rest of the
+// ptl_latent_prepare: per token, from the rows of projections (queries and down-projection, in
+//   one matrix or in two): the RMS norm of the first R entries of the down-projection (float32,
+//   weight w), the rotation of its last dr entries, both written to the cache slot [c | kr]; and
+//   the rotation of the dr rotated entries of every query head, written behind the R entries
+//   that ptl_gemm_heads_nt fills (query rows [H, R + dr]). Rotation of the first 2 * n_pairs
+//   entries, angle = position * inv_freq[i], float32, sine and cosine times ``mag``: neighbouring
+//   pairs (2i, 2i+1), or, with ``half_layout``, entry i with entry i + n_pairs; the rest of the
 //   dr entries pass unchanged.
 // ptl_gemm_heads_nt: out[t, h, :] = x[t, h, :] W_h^T for per-head matrices W [H, N, K], with an
 //   optional factor sigmoid(gate[t, h]) on the result (an output gate per head).
@@ -21,9 +22,10 @@
 
 template <typename T>
 __global__ void __launch_bounds__(256)
-latent_prepare_kernel(T* __restrict__ q_out, long ldq, const T* __restrict__ proj, long ldp, int q_off,
-                      int kv_off, const int32_t* __restrict__ positions, const float* __restrict__ inv_freq,
-                      int n_pairs, const float* __restrict__ c_w, float eps,
+latent_prepare_kernel(T* __restrict__ q_out, long ldq, const T* __restrict__ q_src, long ldqs, int q_off,
+                      const T* __restrict__ kv_src, long ldkv, int kv_off,
+                      const int32_t* __restrict__ positions, const float* __restrict__ inv_freq,
+                      int n_pairs, int half_layout, float mag, const float* __restrict__ c_w, float eps,
                       const int32_t* __restrict__ slots, T* __restrict__ cache, int H, int dn, int dr, int R) {
   extern __shared__ float cs[];          // cos [dr/2], sin [dr/2], scratch [16]
   const int half = dr >> 1;
@@ -34,25 +36,33 @@ latent_prepare_kernel(T* __restrict__ q_out, long ldq, const T* __restrict__ pro
   const float pos = (float)positions[t];
   for (int j = threadIdx.x; j < half; j += 256) {
     float s = 0.f, c = 1.f;
-    if (j < n_pairs) sincosf(pos * inv_freq[j], &s, &c);
+    if (j < n_pairs) {
+      sincosf(pos * inv_freq[j], &s, &c);
+      s *= mag;
+      c *= mag;
+    }
     cosv[j] = c;
     sinv[j] = s;
   }
   __syncthreads();
-  const T* row = proj + (size_t)t * ldp;
+  // the two entries pair j turns: (2j, 2j+1), or (j, j + n_pairs) among the rotating ones of the
+  // half layout (the pairs behind them are the entries that pass)
+  const bool halves = half_layout != 0;
   T* qrow = q_out + (size_t)t * ldq;
   for (int i = threadIdx.x; i < H * half; i += 256) {
     const int h = i / half, j = i - h * half;
-    const T* src = row + q_off + (size_t)h * (dn + dr) + dn + 2 * j;
-    const float u = to_float<T>(src[0]), v = to_float<T>(src[1]);
-    T* dst = qrow + (size_t)h * (R + dr) + R + 2 * j;
-    dst[0] = from_float<T>(u * cosv[j] - v * sinv[j]);
-    dst[1] = from_float<T>(v * cosv[j] + u * sinv[j]);
+    const int a = (halves && j < n_pairs) ? j : 2 * j;
+    const int b = (halves && j < n_pairs) ? j + n_pairs : 2 * j + 1;
+    const T* src = q_src + (size_t)t * ldqs + q_off + (size_t)h * (dn + dr) + dn;
+    const float u = to_float<T>(src[a]), v = to_float<T>(src[b]);
+    T* dst = qrow + (size_t)h * (R + dr) + R;
+    dst[a] = from_float<T>(u * cosv[j] - v * sinv[j]);
+    dst[b] = from_float<T>(v * cosv[j] + u * sinv[j]);
   }
   if (kv_off < 0 || !slots) return;
   const int64_t slot = slots[t];
   if (slot < 0) return;                   // (uniform over the workgroup)
-  const T* d = row + kv_off;
+  const T* d = kv_src + (size_t)t * ldkv + kv_off;
   float ss = 0.f;
   for (int i = threadIdx.x; i < R; i += 256) {
     const float v = to_float<T>(d[i]);
@@ -63,32 +73,39 @@ latent_prepare_kernel(T* __restrict__ q_out, long ldq, const T* __restrict__ pro
   T* dst = cache + (size_t)slot * (R + dr);
   for (int i = threadIdx.x; i < R; i += 256) dst[i] = from_float<T>(to_float<T>(d[i]) * r * c_w[i]);
   for (int j = threadIdx.x; j < half; j += 256) {
-    const float u = to_float<T>(d[R + 2 * j]), v = to_float<T>(d[R + 2 * j + 1]);
-    dst[R + 2 * j] = from_float<T>(u * cosv[j] - v * sinv[j]);
-    dst[R + 2 * j + 1] = from_float<T>(v * cosv[j] + u * sinv[j]);
+    const int a = (halves && j < n_pairs) ? j : 2 * j;
+    const int b = (halves && j < n_pairs) ? j + n_pairs : 2 * j + 1;
+    const float u = to_float<T>(d[R + a]), v = to_float<T>(d[R + b]);
+    dst[R + a] = from_float<T>(u * cosv[j] - v * sinv[j]);
+    dst[R + b] = from_float<T>(v * cosv[j] + u * sinv[j]);
   }
 }
 
-// q_out [T, H, R + dr] (row stride ldq); proj [T, ldp] with the queries [H, dn + dr] from column
-// q_off and the down-projection [R + dr] from column kv_off (kv_off < 0: the layer has none and
-// writes no cache); cache: [slots, R + dr] (pages of one kv head, so slot * (R + dr) is the row);
-// slots null: nothing is written.
-extern "C" int ptl_latent_prepare(void* q_out, long ldq, const void* proj, long ldp, int q_off, int kv_off,
+// q_out [T, H, R + dr] (row stride ldq); q_src [T, ldqs] with the queries [H, dn + dr] from column
+// q_off; kv_src [T, ldkv] (it may be q_src) with the down-projection [R + dr] from column kv_off
+// (kv_off < 0: the layer has none and writes no cache); cache: [slots, R + dr] (pages of one kv
+// head, so slot * (R + dr) is the row); slots null: nothing is written.
+extern "C" int ptl_latent_prepare(void* q_out, long ldq, const void* q_src, long ldqs, int q_off,
+                                  const void* kv_src, long ldkv, int kv_off,
                                   const int32_t* positions, const float* inv_freq, int n_pairs,
+                                  int half_layout, float mag,
                                   const float* c_w, float eps, const int32_t* slots, void* cache,
                                   int T_, int H, int dn, int dr, int R, int dtype, hipStream_t st) {
   if (T_ <= 0) return PTL_OK;
   if (H <= 0 || dn < 0 || dr < 0 || (dr & 1) || R <= 0 || n_pairs < 0 || 2 * n_pairs > dr) return PTL_ERR_ARG;
   if (n_pairs > 0 && !inv_freq) return PTL_ERR_ARG;
+  if (!q_src || (kv_off >= 0 && !kv_src)) return PTL_ERR_ARG;
   if (kv_off >= 0 && slots && (!cache || !c_w)) return PTL_ERR_ARG;
   const size_t lds = (size_t)(dr + 16) * sizeof(float);
   if (dtype == PTL_DTYPE_F32)
-    latent_prepare_kernel<float><<<T_, 256, lds, st>>>((float*)q_out, ldq, (const float*)proj, ldp, q_off,
-                                                       kv_off, positions, inv_freq, n_pairs, c_w, eps, slots,
+    latent_prepare_kernel<float><<<T_, 256, lds, st>>>((float*)q_out, ldq, (const float*)q_src, ldqs, q_off,
+                                                       (const float*)kv_src, ldkv, kv_off, positions, inv_freq,
+                                                       n_pairs, half_layout, mag, c_w, eps, slots,
                                                        (float*)cache, H, dn, dr, R);
   else if (dtype == PTL_DTYPE_BF16)
-    latent_prepare_kernel<bf16_t><<<T_, 256, lds, st>>>((bf16_t*)q_out, ldq, (const bf16_t*)proj, ldp, q_off,
-                                                        kv_off, positions, inv_freq, n_pairs, c_w, eps, slots,
+    latent_prepare_kernel<bf16_t><<<T_, 256, lds, st>>>((bf16_t*)q_out, ldq, (const bf16_t*)q_src, ldqs, q_off,
+                                                        (const bf16_t*)kv_src, ldkv, kv_off, positions,
+                                                        inv_freq, n_pairs, half_layout, mag, c_w, eps, slots,
                                                         (bf16_t*)cache, H, dn, dr, R);
   else
     return PTL_ERR_ARG;

@@ -4,7 +4,10 @@
 //   ptl_moe_topk      per token: scores = sigmoid(logits) or softmax(logits) in float32, the ``top``
 //                     largest (by score plus a per-expert correction, when one is given), their
 //                     experts and scores (the score without the correction is the weight, with or
-//                     without a renormalisation over the chosen ones, times a constant); experts
+//                     without a renormalisation over the chosen ones, times a constant); with
+//                     groups, the experts form equal groups of neighbours, a group's score is the
+//                     sum of its two largest choice scores, and only experts of the best ``keep``
+//                     groups can be chosen; experts
 //                     from ``real`` on have no matrices and return their input: their pairs get
 //                     expert -1 and their weights are added up per token; and the sigmoid of extra
 //                     logit columns behind the experts' (a gate of a shared expert)
@@ -54,8 +57,9 @@ __device__ __forceinline__ float unary_act(int kind, float u) {
 __global__ void __launch_bounds__(256)
 moe_topk_kernel(const float* __restrict__ logits, int ld, int T_, int E, int top, int extra,
                 int renormalize, int score_fn, const float* __restrict__ bias, int real, float renorm_eps,
-                float wscale, int32_t* __restrict__ idx, float* __restrict__ wgt,
-                float* __restrict__ extra_out, float* __restrict__ ident_out) {
+                float wscale, int n_groups, int keep_groups, int32_t* __restrict__ idx,
+                float* __restrict__ wgt, float* __restrict__ extra_out, float* __restrict__ ident_out) {
+  __shared__ float choice[4][64 * TOPK_PER_LANE];      // a token's choice scores (groups only)
   const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
   if (t >= T_) return;
@@ -85,11 +89,58 @@ moe_topk_kernel(const float* __restrict__ logits, int ld, int T_, int E, int top
 #pragma unroll
     for (int i = 0; i < TOPK_PER_LANE; ++i) sc[i] = sigmoidf_(v[i]);
   }
-  if (score_fn == SCORE_SOFTMAX || bias) {
+  if (score_fn == SCORE_SOFTMAX || bias || n_groups > 1) {      // (a group's score sums scores)
 #pragma unroll
     for (int i = 0; i < TOPK_PER_LANE; ++i) {
       const int e = lane + 64 * i;
       if (e < E) v[i] = bias ? sc[i] + bias[e] : sc[i];
+    }
+  }
+  if (n_groups > 1 && keep_groups < n_groups) {
+    // Groups of E / n_groups neighbours; lane g scores group g by its two largest choice scores
+    // (a group of one: by its only one); the best keep_groups groups stay (ties: the lower
+    // group), the choice scores of all others become minus infinity.
+    float* cs = choice[threadIdx.x >> 6];
+#pragma unroll
+    for (int i = 0; i < TOPK_PER_LANE; ++i)
+      if (lane + 64 * i < E) cs[lane + 64 * i] = v[i];
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    const int per = E / n_groups;
+    float gs = -INFINITY;
+    if (lane < n_groups) {
+      float b1 = -INFINITY, b2 = -INFINITY;
+      for (int j = 0; j < per; ++j) {
+        const float x = cs[lane * per + j];
+        if (x > b1) { b2 = b1; b1 = x; }
+        else if (x > b2) b2 = x;
+      }
+      gs = per > 1 ? b1 + b2 : b1;
+    }
+    int kept = 0;
+    for (int k = 0; k < keep_groups; ++k) {
+      float best = gs;
+      int at = gs == -INFINITY ? 0x7fffffff : lane;
+#pragma unroll
+      for (int o = 32; o > 0; o >>= 1) {
+        const float ob = __shfl_xor(best, o, 64);
+        const int oa = __shfl_xor(at, o, 64);
+        if (ob > best || (ob == best && oa < at)) {
+          best = ob;
+          at = oa;
+        }
+      }
+      if (lane == at) {
+        kept = 1;
+        gs = -INFINITY;
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < TOPK_PER_LANE; ++i) {
+      const int e = lane + 64 * i;
+      const int k = __shfl(kept, (e < E ? e / per : 0) & 63, 64);
+      if (e < E && !k) v[i] = -INFINITY;
     }
   }
   float sum = 0.f, ident = 0.f;
@@ -147,17 +198,23 @@ moe_topk_kernel(const float* __restrict__ logits, int ld, int T_, int E, int top
 // the E outputs. bias [E] or null: added to the scores for the choice only. real: the first ``real``
 // outputs are experts with matrices, the others return their input (idx -1; ident_out [T], which
 // must be given when real < E, receives the sum of their weights). Weights: the scores, divided by
-// their sum + renorm_eps when ``renormalize``, times wscale.
+// their sum + renorm_eps when ``renormalize``, times wscale. n_groups > 1: the E outputs form that
+// many equal groups of neighbours (at most 64) of which the best keep_groups can be chosen from.
 extern "C" int ptl_moe_topk(const float* logits, int ld, int T_, int E, int top, int extra, int renormalize,
                             int score_fn, const float* bias, int real, float renorm_eps, float wscale,
-                            int32_t* idx, float* wgt, float* extra_out, float* ident_out, hipStream_t st) {
+                            int n_groups, int keep_groups, int32_t* idx, float* wgt, float* extra_out,
+                            float* ident_out, hipStream_t st) {
   if (T_ <= 0) return PTL_OK;
+  if (n_groups > 1 && (n_groups > 64 || E % n_groups || keep_groups < 1 || keep_groups > n_groups ||
+                       (long)keep_groups * (E / n_groups) < top))
+    return PTL_ERR_ARG;
   if (E <= 0 || top <= 0 || top > E || E > 64 * TOPK_PER_LANE || extra < 0 || extra > 64 || ld < E + extra ||
       (extra && !extra_out) || real < 0 || real > E || (real < E && !ident_out) ||
       (score_fn != SCORE_SIGMOID && score_fn != SCORE_SOFTMAX))
     return PTL_ERR_ARG;
   moe_topk_kernel<<<(T_ + 3) / 4, 256, 0, st>>>(logits, ld, T_, E, top, extra, renormalize, score_fn, bias, real,
-                                                renorm_eps, wscale, idx, wgt, extra_out, ident_out);
+                                                renorm_eps, wscale, n_groups, keep_groups, idx, wgt,
+                                                extra_out, ident_out);
   return ptl_launch_status();
 }
 

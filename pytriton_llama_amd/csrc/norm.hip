@@ -165,6 +165,38 @@ row_scale_kernel(bf16_t* __restrict__ y, const bf16_t* __restrict__ v,
     y[(size_t)m * H + i] = float_to_bf16(bf16_to_float(v[(size_t)m * H + i]) * f);
 }
 
+// RMSNorm of a range of columns of a matrix with strided rows (a slice of a fused projection):
+// y[t, :] = x[t, :] * rsqrt(mean(x[t, :]^2) + eps) * w, H columns, float32 statistics.
+template <typename T>
+__global__ void __launch_bounds__(256)
+rmsnorm_cols_kernel(T* __restrict__ y, long ldy, const T* __restrict__ x, long ldx,
+                    const float* __restrict__ w, int H, float eps) {
+  __shared__ float scratch[16];
+  const T* xr = x + (size_t)blockIdx.x * ldx;
+  T* yr = y + (size_t)blockIdx.x * ldy;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < H; i += 256) {
+    const float v = to_float<T>(xr[i]);
+    ss = fmaf(v, v, ss);
+  }
+  ss = block_sum(ss, scratch);
+  const float rr = 1.0f / sqrtf(ss / (float)H + eps);
+  for (int i = threadIdx.x; i < H; i += 256) yr[i] = from_float<T>(to_float<T>(xr[i]) * rr * w[i]);
+}
+
+extern "C" int ptl_rmsnorm_cols(void* y, long ldy, const void* x, long ldx, const float* w, int T_, int H,
+                                float eps, int dtype, hipStream_t stream) {
+  if (T_ <= 0) return PTL_OK;
+  if (H <= 0 || ldx < H || ldy < H || !w) return PTL_ERR_ARG;
+  if (dtype == PTL_DTYPE_F32)
+    rmsnorm_cols_kernel<float><<<T_, 256, 0, stream>>>((float*)y, ldy, (const float*)x, ldx, w, H, eps);
+  else if (dtype == PTL_DTYPE_BF16)
+    rmsnorm_cols_kernel<bf16_t><<<T_, 256, 0, stream>>>((bf16_t*)y, ldy, (const bf16_t*)x, ldx, w, H, eps);
+  else
+    return PTL_ERR_ARG;
+  return ptl_launch_status();
+}
+
 extern "C" int ptl_row_scale_bf16(void* y, const void* v, const float* partials, int count, int T_,
                                   int H, float eps, hipStream_t stream) {
   if (T_ <= 0) return PTL_OK;

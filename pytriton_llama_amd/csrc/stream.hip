@@ -257,6 +257,41 @@ extern "C" int ptl_embedding_scaled(float* out, const void* table, const int32_t
   return ptl_launch_status();
 }
 
+// out[t] = e * rsqrt(mean(e^2) + eps) * w with e = table[ids[t]] * scale, as float32: a residual
+// stream that starts from the normed embedding, in one pass over the row.
+template <typename T>
+__global__ void __launch_bounds__(256)
+embedding_rmsnorm_kernel(float* __restrict__ out, const T* __restrict__ table, const int32_t* __restrict__ ids,
+                         const float* __restrict__ w, float eps, int H, int V, float scale) {
+  __shared__ float scratch[16];
+  const int t = blockIdx.x;
+  int id = ids[t];
+  if (id < 0 || id >= V) id = 0;          // checked on the host; never read out of bounds
+  const T* src = table + (size_t)id * H;
+  float* dst = out + (size_t)t * H;
+  float ss = 0.f;
+  for (int j = threadIdx.x; j < H; j += 256) {
+    const float v = to_float<T>(src[j]) * scale;
+    ss = fmaf(v, v, ss);
+  }
+  ss = block_sum(ss, scratch);
+  const float r = 1.0f / sqrtf(ss / (float)H + eps);
+  for (int j = threadIdx.x; j < H; j += 256) dst[j] = to_float<T>(src[j]) * scale * r * w[j];
+}
+
+extern "C" int ptl_embedding_rmsnorm(float* out, const void* table, const int32_t* ids, const float* w,
+                                     float eps, int T_, int H, int V, float scale, int dtype, hipStream_t st) {
+  if (T_ <= 0) return PTL_OK;
+  if (H <= 0 || V <= 0 || !w) return PTL_ERR_ARG;
+  if (dtype == PTL_DTYPE_F32)
+    embedding_rmsnorm_kernel<float><<<T_, 256, 0, st>>>(out, (const float*)table, ids, w, eps, H, V, scale);
+  else if (dtype == PTL_DTYPE_BF16)
+    embedding_rmsnorm_kernel<bf16_t><<<T_, 256, 0, st>>>(out, (const bf16_t*)table, ids, w, eps, H, V, scale);
+  else
+    return PTL_ERR_ARG;
+  return ptl_launch_status();
+}
+
 __device__ __forceinline__ float gelu_tanh(float z) {
   return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
 }

@@ -127,6 +127,22 @@ def add_rmsnorm(x: torch.Tensor, residual: Optional[torch.Tensor], weight: torch
     return y
 
 
+def rmsnorm_cols(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+    """rmsnorm(x) * weight for x [T, H] whose rows may be strided (a range of columns of a fused
+    projection); the result is contiguous, in x's dtype. weight is float32 [H]."""
+    _need_gpu(x, weight)
+    if x.dim() != 2 or x.stride(1) != 1:
+        raise KernelError("rmsnorm_cols: x must be a [T, H] matrix with dense rows")
+    T, H = x.shape
+    if weight.dtype != torch.float32 or weight.shape != (H,) or not weight.is_contiguous():
+        raise KernelError(f"rmsnorm_cols: weight must be float32 [{H}]")
+    y = torch.empty((T, H), dtype=x.dtype, device=x.device)
+    _check(library.load("norm").ptl_rmsnorm_cols(_ptr(y), ctypes.c_long(H), _ptr(x),
+                                                 ctypes.c_long(x.stride(0) if T > 1 else H), _ptr(weight), T, H,
+                                                 ctypes.c_float(eps), _dtype_code(x), _stream()), "rmsnorm_cols")
+    return y
+
+
 def silu_mul(gate_up: torch.Tensor) -> torch.Tensor:
     """out[:, i] = silu(gate_up[:, i]) * gate_up[:, I + i] for a [T, 2I] input."""
     _need_gpu(gate_up)
@@ -621,14 +637,28 @@ def qkv_rope_store(x: torch.Tensor, w: torch.Tensor, positions: torch.Tensor,
     return q
 
 
+def _mask_extras(what: str, Hq: int, window: int, keep_first: int, sink: Optional[torch.Tensor]):
+    """The two optional pieces every attention kernel takes: ``keep_first`` (with a window: the
+    keys at positions below it stay visible to every later query) and ``sink`` (float32 [Hq]: the
+    softmax denominator of head h also holds exp(sink[h]), a term without key and value)."""
+    if keep_first < 0 or (keep_first and window <= 0):
+        raise KernelError(f"{what}: keep_first goes with a window, and is not negative")
+    if sink is not None and (not sink.is_cuda or sink.dtype != torch.float32 or sink.shape != (Hq,)
+                             or not sink.is_contiguous()):
+        raise KernelError(f"{what}: sink must be a contiguous float32 GPU tensor [{Hq}]")
+    return int(keep_first), _ptr(sink)
+
+
 def attention_generic(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor,
                       v_cache: torch.Tensor, q_start: torch.Tensor, ctx_len: torch.Tensor,
                       block_table: torch.Tensor, work_seq: torch.Tensor, work_qoff: torch.Tensor,
-                      scale: float, window: int = 0) -> None:
+                      scale: float, window: int = 0, keep_first: int = 0,
+                      sink: Optional[torch.Tensor] = None) -> None:
     """Attention of a mixed batch over the paged cache (see csrc/attention.hip).
     q [T, Hq, D] (rows may be strided), out [T, Hq, D], caches
     [pages, Hkv, page_size, D], q_start [n+1], ctx_len [n], block_table [n, max_pages],
-    work_seq / work_qoff: the list of 16-row query blocks."""
+    work_seq / work_qoff: the list of 16-row query blocks. ``keep_first``, ``sink``: see
+    _mask_extras."""
     _need_gpu(out, q, k_cache, v_cache, q_start, ctx_len, block_table, work_seq, work_qoff)
     T, Hq, D = q.shape
     if k_cache.dim() != 4 or k_cache.shape != v_cache.shape or k_cache.shape[3] != D:
@@ -653,12 +683,13 @@ def attention_generic(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor,
     if block_table.dtype != torch.int32 or block_table.dim() != 2 or block_table.shape[0] < n \
             or block_table.stride(1) != 1:
         raise KernelError("attention: block_table must be int32 [n, max_pages]")
+    keep, sk = _mask_extras("attention", Hq, window, keep_first, sink)
     lib = library.load("attention")
     _check(lib.ptl_attention_generic(
         _ptr(out), ctypes.c_long(out.stride(0)), _ptr(q), ctypes.c_long(q.stride(0)),
         _ptr(k_cache), _ptr(v_cache), _ptr(q_start), _ptr(ctx_len), _ptr(block_table),
         int(block_table.stride(0)), _ptr(work_seq), _ptr(work_qoff), int(work_seq.numel()),
-        Hq, Hkv, D, page_size, int(window), ctypes.c_float(scale), _dtype_code(q), _stream()),
+        Hq, Hkv, D, page_size, int(window), keep, sk, ctypes.c_float(scale), _dtype_code(q), _stream()),
         "attention")
 
 
@@ -695,7 +726,8 @@ def attention_decode_mfma_fits(dtype, Hq: int, Hkv: int, D: int, page_size: int 
 def attention_decode(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor,
                      v_cache: torch.Tensor, q_start: torch.Tensor, ctx_len: torch.Tensor,
                      block_table: torch.Tensor, n_seq: int, scale: float, window: int = 0,
-                     num_splits: int = 1, matrix_cores: bool = False, unroll: int = 0) -> None:
+                     num_splits: int = 1, matrix_cores: bool = False, unroll: int = 0,
+                     keep_first: int = 0, sink: Optional[torch.Tensor] = None) -> None:
     """Split-KV attention of the first ``n_seq`` sequences of the tables, each of
     which brings exactly one query token (see csrc/attention.hip). Head sizes in
     steps of 16 up to 256, float32 or bfloat16. ``matrix_cores``: the MFMA
@@ -710,6 +742,7 @@ def attention_decode(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor,
         raise KernelError("attention_decode: tables are shorter than n_seq")
     if num_splits < 1:
         raise KernelError("attention_decode: num_splits must be >= 1")
+    keep, sk = _mask_extras("attention_decode", Hq, window, keep_first, sink)
     part_acc = part_ml = None
     if num_splits > 1:
         part_acc = torch.empty((n_seq, Hq, num_splits, D), dtype=torch.float32, device=q.device)
@@ -725,14 +758,14 @@ def attention_decode(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor,
             _ptr(out), ctypes.c_long(out.stride(0)), _ptr(q), ctypes.c_long(q.stride(0)),
             _ptr(k_cache), _ptr(v_cache), _ptr(q_start), _ptr(ctx_len), _ptr(block_table),
             int(block_table.stride(0)), _ptr(part_acc), _ptr(part_ml), int(n_seq), Hq, Hkv, D,
-            page_size, int(window), ctypes.c_float(scale), int(num_splits), int(unroll), _stream()),
-            "attention_decode_mfma")
+            page_size, int(window), keep, sk, ctypes.c_float(scale), int(num_splits), int(unroll),
+            _stream()), "attention_decode_mfma")
         return
     _check(lib.ptl_attention_decode(
         _ptr(out), ctypes.c_long(out.stride(0)), _ptr(q), ctypes.c_long(q.stride(0)),
         _ptr(k_cache), _ptr(v_cache), _ptr(q_start), _ptr(ctx_len), _ptr(block_table),
         int(block_table.stride(0)), _ptr(part_acc), _ptr(part_ml), int(n_seq), Hq, Hkv, D, page_size,
-        int(window), ctypes.c_float(scale), int(num_splits), _dtype_code(q), _stream()),
+        int(window), keep, sk, ctypes.c_float(scale), int(num_splits), _dtype_code(q), _stream()),
         "attention_decode")
 
 
@@ -781,7 +814,8 @@ def attention_prefill_mfma(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Te
                            v_cache: torch.Tensor, q_start: torch.Tensor, ctx_len: torch.Tensor,
                            block_table: torch.Tensor, work_seq: torch.Tensor,
                            work_qoff: torch.Tensor, scale: float, window: int = 0,
-                           block_rows: int = 64, groups: int = 0) -> None:
+                           block_rows: int = 64, groups: int = 0, keep_first: int = 0,
+                           sink: Optional[torch.Tensor] = None) -> None:
     """bfloat16 attention of prompt portions on the matrix cores; the work list
     names query blocks of ``block_rows`` (64 or 128) rows, those with the most
     keys first. ``groups`` workgroups a head share the list (0: one for every
@@ -804,6 +838,7 @@ def attention_prefill_mfma(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Te
         raise KernelError("attention_prefill_mfma: query blocks are 64 or 128 rows")
     if q.stride(0) % 8 or out.stride(0) % 4 or q.data_ptr() % 16 or out.data_ptr() % 8:
         raise KernelError("attention_prefill_mfma: q rows must be 16-byte aligned, out rows 8-byte")
+    keep, sk = _mask_extras("attention_prefill_mfma", Hq, window, keep_first, sink)
     lib = library.load("attention_prefill")
     n_work = int(work_seq.numel())
     _check(lib.ptl_attention_prefill_mfma(
@@ -811,7 +846,7 @@ def attention_prefill_mfma(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Te
         _ptr(k_cache), _ptr(v_cache), _ptr(q_start), _ptr(ctx_len), _ptr(block_table),
         int(block_table.stride(0)), _ptr(work_seq), _ptr(work_qoff), n_work,
         min(n_work, int(groups)) if groups > 0 else n_work, int(block_rows), Hq, Hkv, D, page_size,
-        int(window), ctypes.c_float(scale), _stream()), "attention_prefill_mfma")
+        int(window), keep, sk, ctypes.c_float(scale), _stream()), "attention_prefill_mfma")
 
 
 def argmax(logits: torch.Tensor, host_out: Optional[torch.Tensor] = None) -> torch.Tensor:
@@ -958,6 +993,24 @@ def embedding_scaled(table: torch.Tensor, ids: torch.Tensor, scale: float, copie
     return out
 
 
+def embedding_rmsnorm(table: torch.Tensor, ids: torch.Tensor, weight: torch.Tensor, eps: float,
+                      scale: float = 1.0) -> torch.Tensor:
+    """out[t] = rmsnorm(table[ids[t]] * scale) * weight as float32: a float32 residual stream
+    that starts from the normed embedding."""
+    _need_gpu(table, ids, weight)
+    _i32(ids, "ids")
+    if table.dim() != 2 or not table.is_contiguous():
+        raise KernelError("embedding table must be a contiguous [V, H] matrix")
+    V, H = table.shape
+    _f32_vec(weight, H, "embedding_rmsnorm: weight")
+    T = ids.numel()
+    out = torch.empty((T, H), dtype=torch.float32, device=table.device)
+    _check(library.load("stream").ptl_embedding_rmsnorm(_ptr(out), _ptr(table), _ptr(ids), _ptr(weight),
+                                                        ctypes.c_float(eps), T, H, V, ctypes.c_float(scale),
+                                                        _dtype_code(table), _stream()), "embedding_rmsnorm")
+    return out
+
+
 HYPER_MAX_STREAMS = 16
 
 
@@ -1076,19 +1129,26 @@ def gelu_gather_mul(z: torch.Tensor, table: torch.Tensor, ids: torch.Tensor, col
 def latent_prepare(q_out: torch.Tensor, proj: torch.Tensor, q_off: int, kv_off: int,
                    positions: torch.Tensor, inv_freq: Optional[torch.Tensor], c_weight: Optional[torch.Tensor],
                    eps: float, slots: Optional[torch.Tensor], cache: Optional[torch.Tensor],
-                   H: int, dn: int, dr: int, R: int) -> None:
+                   H: int, dn: int, dr: int, R: int, queries: Optional[torch.Tensor] = None,
+                   half_layout: bool = False, mag: float = 1.0) -> None:
     """From the projections ``proj`` [T, >= q_off + H (dn + dr)] of a step: the rotated query
     parts into q_out[:, :, R:] (q_out [T, H, R + dr]), and, when the layer has a down-projection
     (``kv_off`` >= 0: its R + dr columns start there) and ``slots`` are given, the normalised
     latent and the rotated shared key part into ``cache`` [pages, 1, page_size, R + dr] at the
-    tokens' slots. inv_freq float32 [pairs], 2 * pairs <= dr: the entries that rotate."""
-    _need_gpu(q_out, proj, positions, inv_freq, c_weight, slots, cache)
+    tokens' slots. inv_freq float32 [pairs], 2 * pairs <= dr: the entries that rotate, as
+    neighbouring pairs or, with ``half_layout``, entry i with entry i + pairs; sine and cosine
+    times ``mag``. ``queries``: the matrix [T, >= q_off + H (dn + dr)] that holds the queries when
+    they are not columns of ``proj``."""
+    _need_gpu(q_out, proj, positions, inv_freq, c_weight, slots, cache, queries)
     T = proj.shape[0]
     D = R + dr
+    qsrc = proj if queries is None else queries
     if proj.dim() != 2 or proj.stride(1) != 1 or q_out.shape != (T, H, D) or not q_out.is_contiguous() \
             or q_out.dtype != proj.dtype:
         raise KernelError("latent_prepare: proj [T, n] with dense rows, q_out contiguous [T, H, R + dr]")
-    if q_off < 0 or q_off + H * (dn + dr) > proj.shape[1] or (kv_off >= 0 and kv_off + D > proj.shape[1]):
+    if qsrc.dim() != 2 or qsrc.stride(1) != 1 or qsrc.shape[0] != T or qsrc.dtype != proj.dtype:
+        raise KernelError("latent_prepare: queries [T, n] with dense rows, of the projections' dtype")
+    if q_off < 0 or q_off + H * (dn + dr) > qsrc.shape[1] or (kv_off >= 0 and kv_off + D > proj.shape[1]):
         raise KernelError("latent_prepare: the columns named lie outside the projections")
     _i32(positions, "positions")
     if positions.numel() != T or dr % 2:
@@ -1109,8 +1169,10 @@ def latent_prepare(q_out: torch.Tensor, proj: torch.Tensor, q_off: int, kv_off: 
                 or not c_weight.is_contiguous():
             raise KernelError(f"latent_prepare: the latent's norm weight must be float32 [{R}]")
     _check(library.load("latent").ptl_latent_prepare(
-        _ptr(q_out), ctypes.c_long(H * D), _ptr(proj), ctypes.c_long(proj.stride(0)), int(q_off), int(kv_off),
-        _ptr(positions), _ptr(inv_freq), int(pairs), _ptr(c_weight), ctypes.c_float(eps), _ptr(slots),
+        _ptr(q_out), ctypes.c_long(H * D), _ptr(qsrc), ctypes.c_long(qsrc.stride(0)), int(q_off),
+        _ptr(proj), ctypes.c_long(proj.stride(0)), int(kv_off),
+        _ptr(positions), _ptr(inv_freq), int(pairs), int(bool(half_layout)), ctypes.c_float(mag),
+        _ptr(c_weight), ctypes.c_float(eps), _ptr(slots),
         _ptr(cache), T, H, dn, dr, R, _dtype_code(proj), _stream()), "latent_prepare")
 
 
@@ -1144,7 +1206,7 @@ def gemm_heads_nt(out: torch.Tensor, x: torch.Tensor, w: torch.Tensor,
 def attention_generic_kv(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                          q_start: torch.Tensor, ctx_len: torch.Tensor, block_table: torch.Tensor,
                          work_seq: torch.Tensor, work_qoff: torch.Tensor, scale: float, maps: int = 1,
-                         window: int = 0) -> None:
+                         window: int = 0, keep_first: int = 0, sink: Optional[torch.Tensor] = None) -> None:
     """The vector-FMA attention kernel in its general form (csrc/attention.hip): q [T, Hq, Dk]
     with Hq = heads * maps (head after head, map after map), k_cache [pages, Hkv * maps, page_size,
     Dk], v_cache [pages, Hkv, page_size, Dv], out [T, Hq, Dv] in the caches' dtype or float32.
@@ -1176,12 +1238,13 @@ def attention_generic_kv(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tens
     if block_table.dtype != torch.int32 or block_table.dim() != 2 or block_table.shape[0] < n \
             or block_table.stride(1) != 1:
         raise KernelError("attention: block_table must be int32 [n, max_pages]")
+    keep, sk = _mask_extras("attention", Hq, window, keep_first, sink)
     _check(library.load("attention").ptl_attention_generic_kv(
         _ptr(out), ctypes.c_long(out.stride(0)), int(out.dtype == torch.float32 and q.dtype != torch.float32),
         _ptr(q), ctypes.c_long(q.stride(0)), _ptr(k_cache), _ptr(v_cache), _ptr(q_start), _ptr(ctx_len),
         _ptr(block_table), int(block_table.stride(0)), _ptr(work_seq), _ptr(work_qoff),
-        int(work_seq.numel()), Hq, Hkv, int(maps), Dk, Dv, page_size, int(window), ctypes.c_float(scale),
-        _dtype_code(q), _stream()), "attention")
+        int(work_seq.numel()), Hq, Hkv, int(maps), Dk, Dv, page_size, int(window), keep, sk,
+        ctypes.c_float(scale), _dtype_code(q), _stream()), "attention")
 
 
 def attention_prefill_mfma_kv_fits(dtype: torch.dtype, num_kv_heads: int, maps: int, Dk: int, Dv: int,
@@ -1197,7 +1260,8 @@ def attention_prefill_mfma_kv_fits(dtype: torch.dtype, num_kv_heads: int, maps: 
 def attention_prefill_mfma_kv(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                               q_start: torch.Tensor, ctx_len: torch.Tensor, block_table: torch.Tensor,
                               work_seq: torch.Tensor, work_qoff: torch.Tensor, scale: float, maps: int = 1,
-                              groups: int = 1, window: int = 0) -> None:
+                              groups: int = 1, window: int = 0, keep_first: int = 0,
+                              sink: Optional[torch.Tensor] = None) -> None:
     """The matrix-core kernel for prompt portions in its general form (csrc/attention_prefill.hip):
     shapes as for attention_generic_kv, bfloat16 q and caches, out bfloat16 or float32; the work
     list names 64-row blocks, ``groups`` workgroups a head share it."""
@@ -1229,11 +1293,12 @@ def attention_prefill_mfma_kv(out: torch.Tensor, q: torch.Tensor, k_cache: torch
     n_work = int(work_seq.numel())
     if n_work == 0:
         return
+    keep, sk = _mask_extras("attention_prefill_mfma_kv", Hq, window, keep_first, sink)
     _check(library.load("attention_prefill").ptl_attention_prefill_mfma_kv(
         _ptr(out), ctypes.c_long(out.stride(0)), int(out.dtype == torch.float32), _ptr(q),
         ctypes.c_long(q.stride(0)), _ptr(k_cache), _ptr(v_cache), _ptr(q_start), _ptr(ctx_len),
         _ptr(block_table), int(block_table.stride(0)), _ptr(work_seq), _ptr(work_qoff), n_work,
-        max(1, min(int(groups), n_work)), Hq, Hkv, int(maps), Dk, Dv, page_size, int(window),
+        max(1, min(int(groups), n_work)), Hq, Hkv, int(maps), Dk, Dv, page_size, int(window), keep, sk,
         ctypes.c_float(scale), _stream()), "attention_prefill_mfma_kv")
 
 
@@ -1244,7 +1309,8 @@ def attention_decode_kv_fits(Dk: int, Dv: int) -> bool:
 
 def attention_decode_kv(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                         q_start: torch.Tensor, ctx_len: torch.Tensor, block_table: torch.Tensor, n_seq: int,
-                        scale: float, maps: int = 1, num_splits: int = 1, window: int = 0) -> None:
+                        scale: float, maps: int = 1, num_splits: int = 1, window: int = 0,
+                        keep_first: int = 0, sink: Optional[torch.Tensor] = None) -> None:
     """Split-KV attention of the first ``n_seq`` sequences of the tables, each of which brings one
     query token, with keys and values of different sizes and ``maps`` score maps a head (shapes as
     for attention_generic_kv; sizes in steps of 16 up to 256)."""
@@ -1271,6 +1337,7 @@ def attention_decode_kv(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tenso
         raise KernelError("attention_decode_kv: block_table must be int32 [n, max_pages]")
     if n_seq > ctx_len.numel() or q_start.numel() < n_seq + 1 or block_table.shape[0] < n_seq or num_splits < 1:
         raise KernelError("attention_decode_kv: tables are shorter than n_seq, or no splits")
+    keep, sk = _mask_extras("attention_decode_kv", Hq, window, keep_first, sink)
     part_acc = part_ml = None
     if num_splits > 1:
         part_acc = torch.empty((n_seq, Hq, num_splits, Dv), dtype=torch.float32, device=q.device)
@@ -1279,8 +1346,8 @@ def attention_decode_kv(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tenso
         _ptr(out), ctypes.c_long(out.stride(0)), int(out.dtype == torch.float32 and q.dtype != torch.float32),
         _ptr(q), ctypes.c_long(q.stride(0)), _ptr(k_cache), _ptr(v_cache), _ptr(q_start), _ptr(ctx_len),
         _ptr(block_table), int(block_table.stride(0)), _ptr(part_acc), _ptr(part_ml), int(n_seq), Hq, Hkv,
-        int(maps), Dk, Dv, page_size, int(window), ctypes.c_float(scale), int(num_splits), _dtype_code(q),
-        _stream()), "attention_decode_kv")
+        int(maps), Dk, Dv, page_size, int(window), keep, sk, ctypes.c_float(scale), int(num_splits),
+        _dtype_code(q), _stream()), "attention_decode_kv")
 
 
 # ---------------------------------------------------------------------------
@@ -1606,14 +1673,18 @@ class Routing:
 
 def moe_route(logits: torch.Tensor, experts: int, top: int, extra: int = 0,
               renormalize: bool = False, score: int = SCORE_SIGMOID, correction: Optional[torch.Tensor] = None,
-              identity: int = 0, renorm_eps: float = 0.0, weight_scale: float = 1.0) -> Routing:
+              identity: int = 0, renorm_eps: float = 0.0, weight_scale: float = 1.0,
+              groups: int = 1, keep_groups: int = 1) -> Routing:
     """Route every row of float32 ``logits`` [T, experts + identity + extra] to ``top`` of its
     ``experts + identity`` router outputs and order the pairs by expert. Scores: the sigmoid of
     the logits, or their softmax over the router outputs; the choice goes by score +
     ``correction`` [experts + identity] when one is given; the weights are the scores
     (``renormalize``: divided by their sum + renorm_eps) times weight_scale. The last
     ``identity`` outputs are experts that return their input: their pairs take no part in the
-    products, and ``ident`` [T] holds the sum of their weights a token."""
+    products, and ``ident`` [T] holds the sum of their weights a token. ``groups`` > 1: the router
+    outputs form that many equal groups of neighbours (at most 64); a group's score is the sum
+    of its two largest choice scores (score + correction), and only outputs of the best
+    ``keep_groups`` groups can be chosen."""
     _need_gpu(logits)
     if logits.dim() != 2 or logits.dtype != torch.float32 or logits.stride(1) != 1 \
             or logits.shape[1] < experts + extra:
@@ -1626,6 +1697,10 @@ def moe_route(logits: torch.Tensor, experts: int, top: int, extra: int = 0,
                           "kernel takes")
     if correction is not None:
         _f32_vec(correction, outputs, "moe_route: correction")
+    if groups < 1 or (groups > 1 and (groups > 64 or outputs % groups or not 1 <= keep_groups <= groups
+                                      or keep_groups * (outputs // groups) < top)):
+        raise KernelError(f"moe_route: {groups} groups of which {keep_groups} are kept do not fit "
+                          f"{outputs} router outputs with {top} chosen (at most 64 equal groups)")
     T = logits.shape[0]
     A = T * top
     lib = library.load("moe")
@@ -1643,8 +1718,8 @@ def moe_route(logits: torch.Tensor, experts: int, top: int, extra: int = 0,
     r.ident = torch.empty(T, dtype=torch.float32, device=dev) if identity else None
     _check(lib.ptl_moe_topk(_ptr(logits), int(logits.stride(0)), T, outputs, top, extra, int(renormalize),
                             int(score), _ptr(correction), experts, ctypes.c_float(renorm_eps),
-                            ctypes.c_float(weight_scale), _ptr(r.idx), _ptr(r.wgt), _ptr(r.extra),
-                            _ptr(r.ident), _stream()), "moe_topk")
+                            ctypes.c_float(weight_scale), int(groups), int(keep_groups), _ptr(r.idx),
+                            _ptr(r.wgt), _ptr(r.extra), _ptr(r.ident), _stream()), "moe_topk")
     _check(lib.ptl_moe_sort(_ptr(r.idx), A, experts, _ptr(r.pos_of), _ptr(r.sorted), _ptr(r.expert_end),
                             _ptr(r.tile_expert), _ptr(r.tile_row0), r.max_tiles, _stream()), "moe_sort")
     return r

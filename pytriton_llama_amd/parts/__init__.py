@@ -3,7 +3,7 @@ from .base import (PART_KINDS, PART_REGISTRY, PagedSpec, PagedTensor, ParamSourc
                    place, register_part)
 from .linear import linear
 from .norm import DynamicTanh, RMSNorm
-from .rotary import RotaryEncoding, default_inv_freq, llama3_inv_freq, ramp_inv_freq
+from .rotary import RotaryEncoding, banded_inv_freq, default_inv_freq, llama3_inv_freq, ramp_inv_freq
 from .attention import PagedAttention
 from .feedforward import GatedMLP, PlainMLP, RoutedExperts, SwiGLU
 from .latent_attention import LatentAttention

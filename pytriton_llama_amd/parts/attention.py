@@ -50,6 +50,8 @@ class PagedAttention(Part):
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(head_dim)
         self.window = int(window) if window else None
         self.names = (q_name, k_name, v_name, o_name)
+        self.sink: Optional[torch.Tensor] = None    # float32 [heads], set by a mixer that wraps this one:
+                                            # the softmax denominator of head h also holds exp(sink[h])
         self.force_decode_splits = 0        # tests set it to try other splits
         self.q_size = self.num_heads * self.head_dim
         self.kv_size = self.num_kv_heads * self.head_dim
@@ -181,7 +183,8 @@ class PagedAttention(Part):
                     and q.stride(0) % 8 == 0)
             ops.attention_decode(out, q, k, v, ctx.q_start, ctx.ctx_len,
                                  group.block_table, n_dec, self.scale, window,
-                                 self.decode_splits(ctx, n_dec, mfma, q.device), matrix_cores=mfma)
+                                 self.decode_splits(ctx, n_dec, mfma, q.device), matrix_cores=mfma,
+                                 sink=self.sink)
         if n_dec == ctx.num_seqs:
             return
         if (ops.attention_prefill_mfma_fits(q.dtype, self.num_kv_heads, D, cache.page_size)
@@ -192,9 +195,10 @@ class PagedAttention(Part):
                 ctx.work[PORTIONS_128][0].numel(), min(keys, window) if window else keys)
             ws, wo = ctx.work[PORTIONS_128 if rows == 128 else PORTIONS_64]
             ops.attention_prefill_mfma(out, q, k, v, ctx.q_start, ctx.ctx_len,
-                                       group.block_table, ws, wo, self.scale, window, rows, groups)
+                                       group.block_table, ws, wo, self.scale, window, rows, groups,
+                                       sink=self.sink)
         else:
             ws, wo = ctx.work[PORTIONS_16 if n_dec else ALL_16]
             ops.attention_generic(out, q, k, v, ctx.q_start, ctx.ctx_len,
-                                  group.block_table, ws, wo, self.scale, window)
+                                  group.block_table, ws, wo, self.scale, window, sink=self.sink)
 

@@ -97,15 +97,20 @@ class PagedTensor:
 @dataclass(frozen=True)
 class PagedSpec:
     """What a mixer keeps for every token, in pages: any number of named tensors. ``window``:
-    only the last ``window`` positions are ever read again, older pages can be given back.
-    Cache layers with equal specs share a page pool and a block table per request."""
+    only the last ``window`` positions are ever read again, older pages can be given back;
+    ``keep_first``: except the first so many positions of a sequence, which every later query
+    reads (their pages stay). Cache layers with equal specs share a page pool and a block table
+    per request."""
     tensors: Tuple[PagedTensor, ...]
     window: Optional[int] = None
+    keep_first: int = 0
 
     def __post_init__(self):
         names = [t.name for t in self.tensors]
         if not names or len(set(names)) != len(names):
             raise ValueError(f"a paged cache spec needs tensors with names of their own, got {names}")
+        if self.keep_first < 0:
+            raise ValueError("keep_first is a number of positions")
 
 
 def paged_kv_spec(num_kv_heads: int, head_dim: int, window: Optional[int] = None) -> PagedSpec:

@@ -14,11 +14,14 @@ from .linear import LINEAR_LIBRARIES, decode_copy, linear
 class TokenEmbedding(Part):
     """h[t] = E[ids[t]], no scaling (lite_llama/models/llama.py:179,201). With
     ``float32_stream`` the result is E[ids[t]] * scale in float32 whatever the engine's dtype:
-    the start of a residual stream that blocks keep in float32."""
+    the start of a residual stream that blocks keep in float32. ``norm``: an RMS norm part (a
+    weight and an eps; its tensor is named ``norm_name`` behind the table's name) applied to the
+    embedding before anything reads it; the stream then starts from the normed rows."""
     kernel_libraries = ("embedding",)
 
     def __init__(self, vocab_size: int, hidden_size: int, weight_name: str = "weight",
-                 scale: float = 1.0, float32_stream: bool = False, copies: int = 1):
+                 scale: float = 1.0, float32_stream: bool = False, copies: int = 1,
+                 norm: Optional[Part] = None, norm_name: str = ".norm"):
         self.vocab_size, self.hidden_size = int(vocab_size), int(hidden_size)
         self.scale, self.float32_stream = float(scale), bool(float32_stream)
         self.copies = int(copies)           # > 1: a row holds the result that many times (a model
@@ -29,16 +32,29 @@ class TokenEmbedding(Part):
             self.kernel_libraries = ("stream",)
         if self.scale != 1.0 and not self.float32_stream:
             raise ValueError("a scaled embedding is computed into a float32 stream")
+        if norm is not None and (not self.float32_stream or self.copies != 1
+                                 or not (hasattr(norm, "weight") and hasattr(norm, "eps"))):
+            raise ValueError("a norm behind the embedding is an RMS norm (a weight and an eps) and writes "
+                             "one float32 stream")
+        self.norm, self.norm_name = norm, weight_name + norm_name
         self.weight_name = weight_name
         self.weight: Optional[torch.Tensor] = None
 
     def param_sources(self) -> List[ParamSource]:
-        return [ParamSource(self.weight_name, (self.vocab_size, self.hidden_size))]
+        out = [ParamSource(self.weight_name, (self.vocab_size, self.hidden_size))]
+        if self.norm is not None:
+            out += [ParamSource(self.norm_name, s.shape, s.kind, s.init) for s in self.norm.param_sources()]
+        return out
 
     def load(self, tensors, dtype, device) -> None:
         self.weight = place(tensors[self.weight_name], "matrix", dtype, device)
+        if self.norm is not None:
+            (src,) = self.norm.param_sources()
+            self.norm.load({src.name: tensors[self.norm_name]}, dtype, device)
 
     def forward(self, token_ids: torch.Tensor) -> torch.Tensor:
+        if self.norm is not None:           # lookup, statistics and weight in one pass over the row
+            return ops.embedding_rmsnorm(self.weight, token_ids, self.norm.weight, self.norm.eps, self.scale)
         if self.float32_stream:
             return ops.embedding_scaled(self.weight, token_ids, self.scale, self.copies)
         return ops.embedding(self.weight, token_ids)

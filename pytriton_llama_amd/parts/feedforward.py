@@ -149,6 +149,9 @@ class RoutedExperts(Part):
     instead of what it returns. Experts are gated, down(act(gate(x), up(x))) with ``activation``
     "silu" or "clamped", or, with "relu2", down(relu(up(x))^2) without a gate. ``identity``: that
     many router outputs behind the experts' have no tensors; their expert returns its input.
+    ``groups`` = (count, keep): the router outputs form ``count`` equal groups of neighbours; a
+    group's score is the sum of its two largest choice scores (score + correction), and only
+    outputs of the ``keep`` best groups can be chosen (the others count as minus infinity).
     ``shared``: a dense feed-forward that every token runs, added times sigmoid(w_sg . x) when
     ``shared_gate``. The result is float32 (the sum over a token's experts is made there).
     Nothing comes back to the host: routing, the grouping of tokens by expert and the experts'
@@ -163,7 +166,7 @@ class RoutedExperts(Part):
                  activation: str = "clamped", limit: float = 0.0, weight_on_input: bool = True,
                  renormalize: bool = False, shared: Optional[Part] = None, shared_gate: bool = True,
                  score: str = "sigmoid", correction_name: Optional[str] = None, identity: int = 0,
-                 renorm_eps: float = 0.0, route_scale: float = 1.0,
+                 renorm_eps: float = 0.0, route_scale: float = 1.0, groups=None,
                  router_name: str = "router", expert_prefix: str = "e", shared_prefix: str = "shared.",
                  shared_gate_name: str = "shared.sg", gate_name: str = "gate", up_name: str = "up",
                  down_name: str = "down"):
@@ -183,6 +186,12 @@ class RoutedExperts(Part):
         self.weight_on_input, self.renormalize = bool(weight_on_input), bool(renormalize)
         self.score = ops.SCORE_SOFTMAX if score == "softmax" else ops.SCORE_SIGMOID
         self.renorm_eps, self.route_scale = float(renorm_eps), float(route_scale)
+        self.groups, self.keep_groups = (int(groups[0]), int(groups[1])) if groups else (1, 1)
+        outputs = self.num_experts + self.identity
+        if self.groups < 1 or outputs % self.groups or not 1 <= self.keep_groups <= self.groups \
+                or self.keep_groups * (outputs // self.groups) < self.top or self.groups > 64:
+            raise ValueError(f"{self.groups} groups of which {self.keep_groups} are kept do not fit {outputs} "
+                             f"router outputs with {self.top} chosen (at most 64 equal groups)")
         self.correction_name = correction_name
         self.shared = shared
         self.shared_gate = bool(shared_gate) and shared is not None
@@ -237,7 +246,8 @@ class RoutedExperts(Part):
         x = as_tensor(x)
         logits = linear(x, self.router, out_dtype=torch.float32)
         r = ops.moe_route(logits, self.num_experts, self.top, 1 if self.shared_gate else 0, self.renormalize,
-                          self.score, self.correction, self.identity, self.renorm_eps, self.route_scale)
+                          self.score, self.correction, self.identity, self.renorm_eps, self.route_scale,
+                          self.groups, self.keep_groups)
         shared = self.shared.forward(x) if self.shared is not None else None
         return ops.moe_experts(x, r, self.gate_up, self.down, self.act, self.limit, self.weight_on_input,
                                shared, r.extra)

@@ -9,6 +9,7 @@ from .. import ops
 from .attention import PagedAttention
 from .base import PagedSpec, PagedTensor, ParamSource, Part, as_tensor, place, register_part
 from .linear import LINEAR_LIBRARIES, decode_copy, linear
+from .rotary import ramp_inv_freq
 
 
 def paired_inv_freq(base: float, dims: int) -> torch.Tensor:
@@ -34,14 +35,29 @@ class LatentAttention(Part):
 
     ``own_kv`` False: the layer has no down-projection and reads the cache layer another one
     fills (the model's run order hands it that layer, not writable); its kv_rank, rot_dim and
-    rotation are the owner's. ``gated`` False: no output gate. Tensor names are parameters."""
+    rotation are the owner's. ``gated`` False: no output gate. Tensor names are parameters.
+
+    ``q_rank``: the queries pass through a latent of their own, q = W_uq (rmsnorm(W_dq x) w_q)
+    (tensors ``dq_name``, ``q_norm_name``, ``uq_name`` instead of ``q_name``). ``rot_layout``
+    "half": entry i of the rotating entries turns with entry i + rot_dims / 2 instead of its
+    neighbour. ``rot_scaling`` (factor, original, fast, slow): frequencies along a ramp with a
+    factor on sine and cosine (parts/rotary.py: ramp_inv_freq). ``sink_name``: a vector of the
+    checkpoint, one number a head; the softmax denominator of head h also holds exp(sink_h), a
+    term without key and value that the scale does not touch."""
 
     def __init__(self, hidden_size: int, num_heads: int, dim: int, rot_dim: int, vdim: int, kv_rank: int,
                  scale: float, rot_base: float, rot_dims: Optional[int] = None, eps: float = 1e-6,
-                 own_kv: bool = True, gated: bool = True,
+                 own_kv: bool = True, gated: bool = True, q_rank: Optional[int] = None,
+                 rot_layout: str = "pairs", rot_scaling: Optional[dict] = None,
+                 sink_name: Optional[str] = None,
                  q_name: str = "q", dkv_name: str = "dkv", c_norm_name: str = "dkv.norm",
-                 uk_name: str = "uk", uv_name: str = "uv", g_name: str = "g", o_name: str = "o"):
+                 uk_name: str = "uk", uv_name: str = "uv", g_name: str = "g", o_name: str = "o",
+                 dq_name: str = "dq", q_norm_name: str = "dq.norm", uq_name: str = "uq"):
         rot_dims = rot_dim if rot_dims is None else int(rot_dims)
+        if rot_layout not in ("pairs", "half"):
+            raise ValueError(f"unknown layout of the rotating entries {rot_layout!r} (known: 'pairs', 'half')")
+        if q_rank is not None and q_rank <= 0:
+            raise ValueError("the queries' latent has a positive size")
         if rot_dim % 2 or rot_dims % 2 or rot_dims > rot_dim:
             raise ValueError(f"rotated size {rot_dim} with {rot_dims} rotating entries: both must be even, "
                              "the second at most the first")
@@ -51,23 +67,37 @@ class LatentAttention(Part):
         self.dim, self.rot_dim, self.vdim, self.kv_rank = int(dim), int(rot_dim), int(vdim), int(kv_rank)
         self.scale, self.eps = float(scale), float(eps)
         self.own_kv, self.gated = bool(own_kv), bool(gated)
-        self.inv_freq_host = paired_inv_freq(rot_base, rot_dims) if rot_dims else None
+        self.q_rank = int(q_rank) if q_rank else 0
+        self.half_layout = rot_layout == "half"
+        self.mag = 1.0
+        self.inv_freq_host = None
+        if rot_dims and rot_scaling:
+            self.inv_freq_host, self.mag = ramp_inv_freq(
+                rot_base, rot_dims, float(rot_scaling["factor"]), float(rot_scaling["original"]),
+                float(rot_scaling["fast"]), float(rot_scaling["slow"]))
+        elif rot_dims:
+            self.inv_freq_host = paired_inv_freq(rot_base, rot_dims)
         self.inv_freq: Optional[torch.Tensor] = None
-        self.names = dict(q=q_name, dkv=dkv_name, c_norm=c_norm_name, uk=uk_name, uv=uv_name, g=g_name, o=o_name)
+        self.sink_name = sink_name or None
+        self.names = dict(q=q_name, dkv=dkv_name, c_norm=c_norm_name, uk=uk_name, uv=uv_name, g=g_name, o=o_name,
+                          dq=dq_name, q_norm=q_norm_name, uq=uq_name)
         D = self.kv_rank + self.rot_dim
         # the attention itself: the engine's paged attention with one kv head of size D whose
         # keys and values are the same pool
         self.core = PagedAttention(hidden_size, num_heads, 1, D, position=None, scale=self.scale)
         self.q_size = self.num_heads * (self.dim + self.rot_dim)
-        self.kv_off = self.q_size if self.own_kv else -1
-        self.g_off = self.q_size + (D if self.own_kv else 0)
-        self.proj: Optional[torch.Tensor] = None          # rows q | down-projection | gate
+        first = self.q_rank or self.q_size             # the first rows of the fused projection
+        self.kv_off = first if self.own_kv else -1
+        self.g_off = first + (D if self.own_kv else 0)
+        self.proj: Optional[torch.Tensor] = None          # rows q (or its latent) | down-projection | gate
+        self.uq: Optional[torch.Tensor] = None            # [q_size, q_rank], with a latent of the queries
+        self.q_weight: Optional[torch.Tensor] = None
         self.ukT: Optional[torch.Tensor] = None           # [H, kv_rank, dim]
         self.uv: Optional[torch.Tensor] = None            # [H, vdim, kv_rank]
         self.o: Optional[torch.Tensor] = None
         self.c_weight: Optional[torch.Tensor] = None
         self.proj_blocked = self.o_blocked = None
-        libs = ("latent",) + tuple(self.core.kernel_libraries)
+        libs = ("latent", "norm") + tuple(self.core.kernel_libraries)
         self.kernel_libraries = tuple(dict.fromkeys(l for l in libs if l != "rope"))
 
     @property
@@ -90,7 +120,11 @@ class LatentAttention(Part):
 
     def param_sources(self) -> List[ParamSource]:
         n, H, W = self.names, self.num_heads, self.hidden_size
-        out = [ParamSource(n["q"], (self.q_size, W))]
+        if self.q_rank:
+            out = [ParamSource(n["dq"], (self.q_rank, W)), ParamSource(n["q_norm"], (self.q_rank,), "vector"),
+                   ParamSource(n["uq"], (self.q_size, self.q_rank))]
+        else:
+            out = [ParamSource(n["q"], (self.q_size, W))]
         if self.own_kv:
             out += [ParamSource(n["dkv"], (self.kv_rank + self.rot_dim, W)),
                     ParamSource(n["c_norm"], (self.kv_rank,), "vector")]
@@ -98,12 +132,21 @@ class LatentAttention(Part):
                 ParamSource(n["uv"], (H * self.vdim, self.kv_rank))]
         if self.gated:
             out.append(ParamSource(n["g"], (H, W)))
+        if self.sink_name:
+            out.append(ParamSource(self.sink_name, (H,), "vector", init=("normal", 0.0, 1.0)))
         out.append(ParamSource(n["o"], (W, H * self.vdim)))
         return out
 
     def load(self, tensors, dtype, device) -> None:
         n, H = self.names, self.num_heads
-        rows = [tensors[n["q"]]]
+        if self.q_rank:
+            rows = [tensors[n["dq"]]]
+            self.uq = place(tensors[n["uq"]], "matrix", dtype, device)
+            self.q_weight = place(tensors[n["q_norm"]], "vector", dtype, device)
+        else:
+            rows = [tensors[n["q"]]]
+        if self.sink_name:
+            self.core.sink = place(tensors[self.sink_name], "vector", dtype, device)
         if self.own_kv:
             rows.append(tensors[n["dkv"]])
             self.c_weight = place(tensors[n["c_norm"]], "vector", dtype, device)
@@ -133,12 +176,15 @@ class LatentAttention(Part):
         group = ctx.groups[cache.group]
         pool = cache.tensors["latent"]
         p = linear(x, self.proj, blocked=self.proj_blocked)
+        # the queries: columns of the fused projection, or a second product from their normed latent
+        qp = p if not self.q_rank else linear(ops.rmsnorm_cols(p[:, :self.q_rank], self.q_weight, self.eps),
+                                              self.uq)
         q = torch.empty((T, H, D), dtype=x.dtype, device=x.device)
         ops.latent_prepare(q, p, 0, self.kv_off, ctx.positions, self.inv_freq, self.c_weight, self.eps,
                            group.slots if (cache.writable and self.own_kv) else None, pool,
-                           H, self.dim, dr, R)
+                           H, self.dim, dr, R, queries=qp, half_layout=self.half_layout, mag=self.mag)
         if self.dim:
-            qn = p[:, :self.q_size].view(T, H, self.dim + dr)[:, :, :self.dim]
+            qn = qp[:, :self.q_size].view(T, H, self.dim + dr)[:, :, :self.dim]
             ops.gemm_heads_nt(q[:, :, :R], qn, self.ukT)
         else:                               # (queries without an unrotated part: only kr is matched)
             q[:, :, :R].zero_()

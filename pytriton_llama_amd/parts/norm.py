@@ -14,13 +14,16 @@ class RMSNorm(Part):
     """y = (x + residual) * rsqrt(mean((x + residual)^2) + eps) * weight, with the
     sum returned as the new residual (lite_llama/kernels/skip_rmsnorm.py:94-181;
     call sites lite_llama/models/llama.py:149,160,219). Without a residual the
-    input itself is the residual (:181)."""
+    input itself is the residual (:181). ``offset``: what is added to the checkpoint's vector
+    to give the weight (1.0 for a design that stores its norm weights around zero)."""
     kernel_libraries = ("norm", "gemm", "gemm_rows", "stream")
     takes_pending_product = True
 
-    def __init__(self, size: int, eps: float, weight_name: str = "weight", streams: int = 1):
+    def __init__(self, size: int, eps: float, weight_name: str = "weight", streams: int = 1,
+                 offset: float = 0.0):
         self.size = int(size)
         self.eps = float(eps)
+        self.offset = float(offset)
         self.streams = int(streams)         # > 1: the rows hold that many float32 streams side by
                                             # side, and their sum is what is normed
         self.weight_name = weight_name
@@ -28,10 +31,13 @@ class RMSNorm(Part):
         self.dtype: Optional[torch.dtype] = None
 
     def param_sources(self) -> List[ParamSource]:
-        return [ParamSource(self.weight_name, (self.size,), "vector")]
+        init = ("normal", 0.0, 0.1) if self.offset else None      # (random weights: around 1 - offset)
+        return [ParamSource(self.weight_name, (self.size,), "vector", init=init)]
 
     def load(self, tensors, dtype, device) -> None:
         self.weight = place(tensors[self.weight_name], "vector", dtype, device)
+        if self.offset:
+            self.weight = self.weight + self.offset
         self.dtype = dtype
 
     def forward(self, x, residual: Optional[torch.Tensor], scale_ok: bool = False):

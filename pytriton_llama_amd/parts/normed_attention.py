@@ -11,7 +11,7 @@ from .. import ops
 from .attention import ALL_16, PORTIONS_16, PORTIONS_64
 from .base import PagedSpec, PagedTensor, ParamSource, Part, PendingSum, as_tensor, place, register_part
 from .linear import LINEAR_LIBRARIES, decode_copy, linear
-from .rotary import ramp_inv_freq
+from .rotary import banded_inv_freq, ramp_inv_freq
 
 
 def pad_rows(rows: torch.Tensor, multiple: int = 8) -> torch.Tensor:
@@ -33,7 +33,11 @@ class NormedAttention(Part):
                 entries of every head (entry i with i + rot_dims / 2) by position * frequency
         a_m = softmax_j<=i (q_m(i) . k_m(j) * scale) v(j)         one result a map, same values
                 (``window``: over the keys with i - j < window only, the query's own and the
-                window - 1 before it; pages that every later query has left behind are given back)
+                window - 1 before it; pages that every later query has left behind are given back.
+                ``keep_first``: and over the keys at positions below it, which stay where they
+                are and are never given back. ``sink_name``: a vector of the checkpoint, one
+                number a head; the softmax denominator of head h also holds exp(sink_h), a term
+                without key and value that the scale does not touch)
 
     maps = 1: out = W_o concat_h a + b_o.
     maps = 2 (differential attention: the second map is subtracted so that what both maps give
@@ -47,13 +51,17 @@ class NormedAttention(Part):
     cache layer of another one (the run order hands it over, not writable); sizes and rotation
     are the owner's. Scores, softmax, norms, angles and lam are float32; the projection's result is
     taken in float32 so that bias and norm see it unrounded. Tensor names are parameters; biases
-    are the projection's name with ".b" added."""
+    are the projection's name with ".b" added. ``rot_scaling``: None, or the numbers of a
+    frequency scaling: factor, original, fast, slow (a ramp between the entries that turn fast and
+    slow, parts/rotary.py: ramp_inv_freq, with its factor on sine and cosine) or factor, original,
+    low, high (by wavelength band, banded_inv_freq)."""
 
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, dim: int, vdim: int,
                  scale: Optional[float] = None, eps: float = 1e-6, qk_norm: Optional[str] = "head",
                  maps: int = 1, diff: float = 0.0, bias: bool = True, gated: bool = False,
                  rot_dims: int = 0, rot_base: float = 10000.0, rot_scaling: Optional[dict] = None,
-                 own_kv: bool = True, window: Optional[int] = None, q_name: str = "q", k_name: str = "k", v_name: str = "v",
+                 own_kv: bool = True, window: Optional[int] = None, keep_first: int = 0,
+                 sink_name: Optional[str] = None, q_name: str = "q", k_name: str = "k", v_name: str = "v",
                  g_name: str = "g", o_name: str = "o", lambda_names=("lq1", "lk1", "lq2", "lk2")):
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} heads are not a multiple of {num_kv_heads} kv heads")
@@ -78,10 +86,21 @@ class NormedAttention(Part):
         if window is not None and window <= 0:
             raise ValueError("a window holds at least the query's own position")
         self.window = int(window) if window else None
+        if keep_first < 0 or (keep_first and not self.window):
+            raise ValueError("first positions are kept beside a window, and their number is not negative")
+        self.keep_first = int(keep_first)
+        if sink_name and maps != 1:
+            raise ValueError("a term of the denominator without a key is built for one score map a head")
+        self.sink_name = sink_name or None
+        self.sink = None
         self.mag = 1.0
         self.inv_freq_host = None
         if self.rot_dims:
-            if rot_scaling:
+            if rot_scaling and "low" in rot_scaling:
+                self.inv_freq_host = banded_inv_freq(
+                    rot_base, self.rot_dims, float(rot_scaling["factor"]), float(rot_scaling["low"]),
+                    float(rot_scaling["high"]), float(rot_scaling["original"]))
+            elif rot_scaling:
                 self.inv_freq_host, self.mag = ramp_inv_freq(
                     rot_base, self.rot_dims, float(rot_scaling["factor"]), float(rot_scaling["original"]),
                     float(rot_scaling["fast"]), float(rot_scaling["slow"]))
@@ -120,7 +139,7 @@ class NormedAttention(Part):
             return self.force_decode_splits
         span = max(ctx.ctx_lens[:n_dec])
         if self.window:
-            span = min(span, self.window)
+            span = min(span, self.window + self.keep_first)
         cus = ops.compute_units(device)
         if matrix_cores:
             base = max(1, n_dec * self.num_kv_heads)
@@ -142,6 +161,7 @@ class NormedAttention(Part):
         16-row blocks."""
         n_dec = ctx.num_decode_seqs if ops.attention_decode_kv_fits(self.dim, self.vdim) else 0
         window = self.window or 0
+        extras = dict(keep_first=self.keep_first, sink=self.sink)
         # one map and keys as large as values: the matrix-core form of the split-KV kernel takes them
         mfma = (n_dec and self.maps == 1 and self.dim == self.vdim and q.stride(0) % 8 == 0
                 and ops.attention_decode_mfma_fits(q.dtype, self.num_heads, self.num_kv_heads, self.dim,
@@ -149,10 +169,11 @@ class NormedAttention(Part):
         if mfma:
             ops.attention_decode(a, q, cache.k, cache.v, ctx.q_start, ctx.ctx_len, group.block_table, n_dec,
                                  self.scale, window, self.decode_splits(ctx, n_dec, q.device, True),
-                                 matrix_cores=True)
+                                 matrix_cores=True, **extras)
         elif n_dec:
             ops.attention_decode_kv(a, q, cache.k, cache.v, ctx.q_start, ctx.ctx_len, group.block_table, n_dec,
-                                    self.scale, self.maps, self.decode_splits(ctx, n_dec, q.device), window)
+                                    self.scale, self.maps, self.decode_splits(ctx, n_dec, q.device), window,
+                                    **extras)
         if n_dec == ctx.num_seqs:
             return
         if n_dec == ctx.num_decode_seqs and ops.attention_prefill_mfma_kv_fits(
@@ -164,17 +185,18 @@ class NormedAttention(Part):
             blocks = ws.numel()
             ops.attention_prefill_mfma_kv(a, q, cache.k, cache.v, ctx.q_start, ctx.ctx_len, group.block_table,
                                           ws, wo, self.scale, self.maps, blocks if blocks <= 2 * t else t,
-                                          window)
+                                          window, **extras)
             return
         ws, wo = ctx.work[PORTIONS_16 if n_dec else ALL_16]
         ops.attention_generic_kv(a, q, cache.k, cache.v, ctx.q_start, ctx.ctx_len, group.block_table,
-                                 ws, wo, self.scale, self.maps, window)
+                                 ws, wo, self.scale, self.maps, window, **extras)
 
     def cache_spec(self):
         if not self.own_kv:
             return None
         return PagedSpec((PagedTensor("k", (self.num_kv_heads * self.maps, self.dim), 1),
-                          PagedTensor("v", (self.num_kv_heads, self.vdim), 1)), self.window)
+                          PagedTensor("v", (self.num_kv_heads, self.vdim), 1)), self.window,
+                         self.keep_first)
 
     def _norm_sizes(self):
         if self.norm_mode == ops.NORM_WHOLE:
@@ -202,6 +224,8 @@ class NormedAttention(Part):
             out += [ParamSource(x, (self.dim,), "vector", init=("normal", 0.0, 0.1)) for x in self.lambda_names]
         if self.gated:
             out.append(ParamSource(n["g"], (self.o_size, W)))
+        if self.sink_name:
+            out.append(ParamSource(self.sink_name, (self.num_heads,), "vector", init=("normal", 0.0, 1.0)))
         out.append(ParamSource(n["o"], (W, self.o_size)))
         if self.bias:
             out.append(ParamSource(n["o"] + ".b", (W,), "vector", init=small))
@@ -231,6 +255,8 @@ class NormedAttention(Part):
             self.lam = float(torch.exp((lq1 * lk1).sum()) - torch.exp((lq2 * lk2).sum())) + self.diff
         if self.inv_freq_host is not None:
             self.inv_freq = self.inv_freq_host.to(device)
+        if self.sink_name:
+            self.sink = place(tensors[self.sink_name], "vector", dtype, device)
 
     def make_decode_copies(self) -> int:
         self.proj_blocked, self.o_blocked = decode_copy(self.proj), decode_copy(self.o)

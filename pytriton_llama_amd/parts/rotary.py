@@ -33,6 +33,21 @@ def llama3_inv_freq(theta: float, dim: int, factor: float, low_freq_factor: floa
     return torch.where(medium, blended, scaled)
 
 
+def banded_inv_freq(base: float, dims: int, factor: float, low: float, high: float, original: float):
+    """f_i = base^(-2i/dims) rescaled by wavelength band, as Llama 3.1 does it: with l = 2 pi / f,
+    waves shorter than original / high keep f, waves longer than original / low get f / factor,
+    those between get (1 - s) f / factor + s f with s = (original / l - low) / (high - low).
+    Worked out in float64, rounded once; float32 [dims / 2]. (llama3_inv_freq above is the same
+    rule in the float32 arithmetic of the reference.)"""
+    i = torch.arange(0, dims // 2, dtype=torch.float64)
+    f = float(base) ** (-2.0 * i / dims)
+    wave = 2.0 * math.pi / f
+    s = (original / wave - low) / (high - low) if high != low else torch.ones_like(f)
+    blend = (1.0 - s) * f / factor + s * f
+    out = torch.where(wave < original / high, f, torch.where(wave > original / low, f / factor, blend))
+    return out.to(torch.float32)
+
+
 def ramp_inv_freq(base: float, dims: int, factor: float, original: float, fast: float, slow: float):
     """Frequencies that go over from the unscaled f_i = base^(-2i/dims) (fast entries) to f_i /
     factor (slow entries) along a linear ramp, and the factor on sine and cosine that goes with
