@@ -25,7 +25,7 @@ ROUND_TO = None
 # choice of groups or of experts (the gap between the last taken and the first left out is below
 # CLOSE_CALL times the size of the two).
 ROUTER_MARGINS = None
-CLOSE_CALL = 0.05
+CLOSE_CALL = 0.02
 
 
 def stored(x):
@@ -242,9 +242,12 @@ def sub(tensors, prefix):
     return {k[len(prefix):]: v for k, v in tensors.items() if k.startswith(prefix)}
 
 
-def forward(cfg, tensors, tokens, dtype=torch.float64, layers_out=None):
-    """Logits [T, vocab] of one whole sequence. ``layers_out``: a list that receives the residual
-    stream behind every layer."""
+def forward(cfg, tensors, tokens, round_to=None, dtype=torch.float64, layers_out=None):
+    """Logits [T, vocab] of one whole sequence. ``round_to``: the dtype an engine stores its
+    intermediate results in (they are rounded to it where an engine rounds). ``layers_out``: a
+    list that receives the residual stream behind every layer."""
+    global ROUND_TO
+    ROUND_TO = round_to
     t = {k: (v.to(dtype) if v.is_floating_point() else v) for k, v in tensors.items()}
     eps = float(cfg["norm"]["eps"])
     tokens = torch.as_tensor(tokens, dtype=torch.long)

@@ -1,0 +1,126 @@
+"""Small Senavik configurations for the tests, none of them anyone's model. Between them they vary
+every size and every branch: both mixers first and last; windows of 1, shorter and longer than a
+page, longer than any test sequence, and none; 0 to 17 kept first tokens (none, fewer than a page,
+exactly a page, more than a page, more than the window); rotations of a whole head, of a part and
+none, with and without rescaled frequencies, with band edges and ramps that meet all their
+branches (also a ramp whose ends coincide); one to four heads a kv head; key and value sizes that
+are equal, that differ either way and that are no multiple of 16; latents whose size with the
+rotated part is 24, 32, 40, 64 and 96 (so the vector, split-KV and matrix-core kernels are all
+met); query latents smaller and larger than the width; dense, routed and absent feed-forwards;
+experts in 1 to 6 groups of 1 to 4 of which 1 to all are kept, and no groups entry; 1 to 3
+experts a token."""
+import copy
+
+
+def attention(heads, kv_heads, dim, vdim, scale, window=None, keep_first=None, rot=None, scaling=None):
+    m = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": scale}
+    if window is not None:
+        m["mask"] = {"size": window}
+        if keep_first is not None:
+            m["mask"]["keep_first"] = keep_first
+    if rot is not None:
+        m["rot"] = {"base": rot[0], "dims": rot[1]}
+        if scaling is not None:
+            m["rot"]["scaling"] = dict(zip(("factor", "low", "high", "original"), scaling))
+    return "attention", m
+
+
+def latent(heads, dim, rot_dim, vdim, kv_rank, q_rank, scale, rot, scaling=None):
+    m = {"heads": heads, "dim": dim, "rot_dim": rot_dim, "vdim": vdim, "kv_rank": kv_rank, "q_rank": q_rank,
+         "scale": scale, "rot": {"base": rot[0], "dims": rot[1]}}
+    if scaling is not None:
+        m["rot"]["scaling"] = dict(zip(("factor", "original", "fast", "slow"), scaling))
+    return "latent_attention", m
+
+
+def dense(ff):
+    return {"kind": "dense", "ff": ff}
+
+
+def moe(ff, experts, top, groups=None):
+    r = {"experts": experts, "top": top}
+    if groups is not None:
+        r["groups"] = {"count": groups[0], "keep": groups[1]}
+    return {"kind": "moe", "expert": {"ff": ff}, "router": r}
+
+
+def layer(kind_mixer, mlp):
+    kind, m = kind_mixer
+    return {"type": kind, "mixer": m, "mlp": mlp}
+
+
+def model(vocab, width, eps, layers):
+    return {"architecture": "Senavik", "vocab": vocab, "width": width, "norm": {"eps": eps}, "layers": layers}
+
+
+def _s1():
+    """Pages of 4. A window of 20 that keeps 3 tokens (less than a page); frequencies in all three
+    bands; a latent of 20 + 12 = 32 (the matrix-core kernels) with a ramp of two branches; eight
+    experts in four pairs of which two are kept; a layer without a feed-forward."""
+    a = attention(4, 2, 16, 24, 0.3, window=20, keep_first=3, rot=(10000.0, 8), scaling=(4.0, 1.0, 4.0, 64))
+    l = latent(3, 8, 12, 12, 20, 16, 0.25, rot=(5000.0, 12), scaling=(4.0, 32, 8.0, 1.0))
+    return model(200, 64, 1e-5, [
+        layer(a, moe(40, 8, 2, groups=(4, 2))),
+        layer(l, dense(48)),
+        layer(a, None),
+        layer(l, moe(32, 6, 3, groups=(3, 2))),
+    ])
+
+
+def _s2():
+    """Pages of 8. The latent mixer first and last; attention without a window, and without a
+    rotation; a window without kept tokens; no groups entry; one expert a token; sizes that are
+    no multiple of 16 (latent 18 + 6 = 24: the vector kernel alone); a rotation of part of the
+    rotated entries; a query latent larger than the width; a ramp whose ends coincide."""
+    return model(150, 72, 1e-6, [
+        layer(latent(2, 10, 6, 14, 18, 80, 0.3, rot=(800.0, 4), scaling=(8.0, 32, 64.0, 16.0)), moe(36, 3, 1)),
+        layer(attention(3, 3, 12, 20, 0.25), None),
+        layer(attention(6, 2, 20, 12, 0.2, window=7, rot=(500.0, 20)), moe(24, 6, 2, groups=(1, 1))),
+        layer(latent(5, 6, 8, 8, 32, 24, 0.35, rot=(10000.0, 8)), dense(40)),
+    ])
+
+
+def _s3():
+    """Pages of 16. Sizes the matrix-core and split-KV kernels take: keys of 32 with values of 64,
+    keys and values of 64 with two heads a kv head; windows of 33 and 40 that keep 17 (more than a
+    page) and 16 (a page); a latent of 48 + 16 = 64; six experts in three pairs, two pairs kept,
+    three experts a token."""
+    return model(180, 96, 1e-5, [
+        layer(attention(4, 2, 32, 64, 0.2, window=33, keep_first=17, rot=(10000.0, 32), scaling=(8.0, 1.0, 4.0, 128)),
+              moe(64, 6, 3, groups=(3, 2))),
+        layer(latent(4, 16, 16, 32, 48, 40, 0.2, rot=(20000.0, 16), scaling=(2.0, 64, 16.0, 2.0)), dense(64)),
+        layer(attention(4, 2, 64, 64, 0.15, window=40, keep_first=16, rot=(2000.0, 16)), moe(48, 4, 2, groups=(2, 1))),
+        layer(latent(2, 32, 32, 64, 64, 32, 0.15, rot=(10000.0, 32)), None),
+    ])
+
+
+def _s4():
+    """Attention layers only (windows of 48 and 24 over pages of 8 that keep 5 and 8 tokens, and
+    one without a window): what a key does to the logits is the attention's doing alone."""
+    return model(200, 64, 1e-5, [
+        layer(attention(4, 2, 32, 32, 0.18, window=48, keep_first=5, rot=(10000.0, 32)), dense(48)),
+        layer(attention(2, 1, 16, 48, 0.25, window=24, keep_first=8, rot=(800.0, 8), scaling=(4.0, 1.0, 2.0, 40)), None),
+        layer(attention(4, 4, 32, 32, 0.18, rot=(10000.0, 16)), moe(48, 4, 1, groups=(4, 2))),
+    ])
+
+
+def _s5():
+    """Pages of 4. A window of one (a query sees itself and the kept tokens), kept tokens beyond
+    the window, a window longer than any test sequence, one head, four heads a kv head, groups of
+    one expert, every group kept, a latent of 32 + 8 = 40 (split-KV and vector kernels)."""
+    return model(120, 48, 1e-4, [
+        layer(attention(2, 1, 8, 8, 0.35, window=1, keep_first=2), moe(24, 4, 2, groups=(4, 3))),
+        layer(latent(1, 8, 8, 16, 32, 12, 0.3, rot=(10000.0, 8), scaling=(4.0, 16, 4.0, 1.0)), None),
+        layer(attention(4, 1, 24, 40, 0.2, window=6, keep_first=9, rot=(10000.0, 24)), moe(24, 3, 2, groups=(3, 3))),
+        layer(attention(1, 1, 16, 16, 0.3, window=4000, keep_first=4, rot=(100.0, 16)), dense(32)),
+    ])
+
+
+# name -> (config, weight std, page size)
+SENAVIK = {"S1": (_s1(), 0.12, 4), "S2": (_s2(), 0.15, 8), "S3": (_s3(), 0.12, 16), "S4": (_s4(), 0.12, 8),
+           "S5": (_s5(), 0.15, 4)}
+
+
+def senavik(name):
+    cfg, std, page = SENAVIK[name]
+    return copy.deepcopy(cfg), std, page
