@@ -309,6 +309,42 @@ MATUSUN_SIZES = {
 }
 
 
+def senavik_shape(width, layers, heads, kv_heads, dim, window, keep_first, latent_heads, latent_dim, rot_dim,
+                  latent_vdim, kv_rank, q_rank, dense_ff, experts, groups, keep_groups, top, expert_ff, vocab):
+    """A Senavik config.json of a real model's layer sizes: windowed attention that keeps the first
+    tokens and latent attention in turn, the first layer with a dense feed-forward, the others
+    routed (experts in groups)."""
+    attn = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5,
+            "mask": {"size": window, "keep_first": keep_first},
+            "rot": {"base": 500000.0, "dims": dim // 2,
+                    "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}}
+    lat = {"heads": latent_heads, "dim": latent_dim, "rot_dim": rot_dim, "vdim": latent_vdim, "kv_rank": kv_rank,
+           "q_rank": q_rank, "scale": (latent_dim + rot_dim) ** -0.5,
+           "rot": {"base": 10000.0, "dims": rot_dim,
+                   "scaling": {"factor": 40.0, "original": 4096, "fast": 32.0, "slow": 1.0}}}
+    moe = {"kind": "moe", "expert": {"ff": expert_ff},
+           "router": {"experts": experts, "top": top, "groups": {"count": groups, "keep": keep_groups}}}
+    out = [{"type": "attention" if i % 2 == 0 else "latent_attention", "mixer": attn if i % 2 == 0 else lat,
+            "mlp": {"kind": "dense", "ff": dense_ff} if i == 0 else moe} for i in range(layers)]
+    return {"architecture": "Senavik", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "layers": out,
+            "initializer_range": 0.02}
+
+
+# name -> (Senavik sizes, the Llama shape of equal width, depth, heads and feed-forward width a token)
+SENAVIK_SIZES = {
+    "2048": (dict(width=2048, layers=8, heads=16, kv_heads=4, dim=128, window=1024, keep_first=4, latent_heads=16,
+                  latent_dim=64, rot_dim=32, latent_vdim=64, kv_rank=96, q_rank=768, dense_ff=8192, experts=16,
+                  groups=4, keep_groups=2, top=2, expert_ff=4096, vocab=32000),
+             dict(num_hidden_layers=8, hidden_size=2048, num_attention_heads=16, num_key_value_heads=4,
+                  head_dim=128, intermediate_size=8192, vocab_size=32000, tie_word_embeddings=False)),
+    "4096": (dict(width=4096, layers=4, heads=32, kv_heads=8, dim=128, window=2048, keep_first=4, latent_heads=32,
+                  latent_dim=64, rot_dim=32, latent_vdim=64, kv_rank=96, q_rank=1536, dense_ff=14336, experts=32,
+                  groups=8, keep_groups=4, top=4, expert_ff=3584, vocab=32000),
+             dict(num_hidden_layers=4, hidden_size=4096, num_attention_heads=32, num_key_value_heads=8,
+                  head_dim=128, intermediate_size=14336, vocab_size=32000, tie_word_embeddings=False)),
+}
+
+
 def engine_rates(cfg, dtype, S, batch, steps, warmup):
     """Prefill of one S-token prompt (one step) and decode steps of ``batch`` requests behind
     S-token prompts, through the whole engine, for any architecture."""
@@ -364,10 +400,11 @@ def _tensors_of(model):
     return [torch.empty(src.shape, device="meta") for _, src in model.expected_tensors().values()]
 
 
-def beside_llama(args, design, wanted, models, sizes_table, shape):
+def beside_llama(args, design, wanted, models, sizes_table, shape, others=()):
     """Prefill and decode throughput of another design at layer sizes of real models, beside the
     Llama decoder of equal width, depth and feed-forward width a token, same engine, same
-    measurement. One JSON line."""
+    measurement. ``others``: (label, sizes table, shape function) of further designs to run at
+    the same named sizes. One JSON line."""
     rows = {}
     for name in [n for n in wanted.split(",") if n]:
         if name not in sizes_table:
@@ -376,7 +413,8 @@ def beside_llama(args, design, wanted, models, sizes_table, shape):
         d_sizes, l_shape = sizes_table[name]
         llama = dict(LLAMA_1B)
         llama.update(l_shape)
-        for label, cfg in ((design, shape(**d_sizes)), ("llama", llama)):
+        beside = [(label, fn(**table[name][0])) for label, table, fn in others if name in table]
+        for label, cfg in [(design, shape(**d_sizes))] + beside + [("llama", llama)]:
             if label not in models.split(","):
                 continue
             log(f"width {name}: {label}")
@@ -402,6 +440,13 @@ def virusun_beside_llama(args):
 
 def matusun_beside_llama(args):
     return beside_llama(args, "matusun", args.matusun, args.matusun_models, MATUSUN_SIZES, matusun_shape)
+
+
+def senavik_beside_llama(args):
+    """Senavik beside Llama and, with 'matusun' among --senavik-models, beside the design whose
+    layers are closest to its own (windowed attention, routed experts, a float32 stream)."""
+    return beside_llama(args, "senavik", args.senavik, args.senavik_models, SENAVIK_SIZES, senavik_shape,
+                        others=(("matusun", MATUSUN_SIZES, matusun_shape),))
 
 
 def main():
@@ -447,6 +492,11 @@ def main():
                     help="the same for the Matusun design (sizes of: 2048, 4096)")
     ap.add_argument("--matusun-models", default="matusun,llama",
                     help="with --matusun: which of the two models to run (for profiles of one of them)")
+    ap.add_argument("--senavik", default="", metavar="SIZES",
+                    help="the same for the Senavik design (sizes of: 2048, 4096)")
+    ap.add_argument("--senavik-models", default="senavik,llama",
+                    help="with --senavik: which models to run, of senavik, llama and matusun (the design with "
+                         "the closest layers, at the same named size)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU: this engine has no multi-GPU path, --gpus {args.gpus} is not run")
@@ -477,6 +527,8 @@ def main():
         return virusun_beside_llama(args)
     if args.matusun:
         return matusun_beside_llama(args)
+    if args.senavik:
+        return senavik_beside_llama(args)
     if args.mixed:
         return mixed_workload(args, cfg, short)
     if args.like_reference:
