@@ -629,7 +629,8 @@ __device__ __forceinline__ void wave_lds_fence() {
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
-template <int NDT, int UNR>
+// KEPT: a window that keeps the sequence's first keys (keep_first > 0).
+template <int NDT, int UNR, bool KEPT>
 __global__ void __launch_bounds__(256)
 attn_decode_mfma_kernel(bf16_t* __restrict__ out, long out_stride, const bf16_t* __restrict__ q,
                         long q_stride, const bf16_t* __restrict__ k_cache,
@@ -654,14 +655,14 @@ attn_decode_mfma_kernel(bf16_t* __restrict__ out, long out_stride, const bf16_t*
   const int k_lo = window > 0 ? max(0, ctx - window) : 0;
   // the walk: the kept first keys left of the window, then the window; k_begin, k_end and the
   // keys of a turn are indices of the walk, key_at gives the position
-  const int n_kept = min(max(keep_first, 0), k_lo);
+  const int n_kept = KEPT ? min(max(keep_first, 0), k_lo) : 0;
   const int shift = k_lo - n_kept;
   const int span = ctx - shift;
   const int per_split = ((span + num_splits - 1) / num_splits + TILE - 1) / TILE * TILE;
   const int k_begin = split * per_split;
   const int k_end = min(span, k_begin + per_split);
   const int turns = (k_end - k_begin + TILE - 1) / TILE;
-  auto key_at = [&](int kw) { return kw < n_kept ? kw : kw + shift; };
+  auto key_at = [&](int kw) { return (KEPT && kw < n_kept) ? kw : kw + shift; };
   const int32_t* bt = block_table + (size_t)seq * bt_stride;
   const uint32_t page_bytes = (uint32_t)Hkv * page_size * D * 2;
   const int page_mask = page_size - 1;
@@ -862,10 +863,16 @@ static int launch_decode_mfma(void* out, long out_stride, const void* q, long q_
   const size_t lds_merge = (size_t)(4 * 16 * D + 4 * 16 * 2) * sizeof(float);
   const size_t lds_values = (size_t)4 * UNR * 16 * (D + 16) * sizeof(bf16_t);
   const size_t lds = lds_merge > lds_values ? lds_merge : lds_values;
-  attn_decode_mfma_kernel<NDT, UNR><<<grid, 256, lds, stream>>>(
-      (bf16_t*)out, out_stride, (const bf16_t*)q, q_stride, (const bf16_t*)k_cache,
-      (const bf16_t*)v_cache, q_start, ctx_len, block_table, bt_stride, part_acc, part_ml, Hq, Hkv,
-      page_size, page_shift, window, keep_first, sink, scale * 1.4426950408889634f, num_splits);
+  if (window > 0 && keep_first > 0)
+    attn_decode_mfma_kernel<NDT, UNR, true><<<grid, 256, lds, stream>>>(
+        (bf16_t*)out, out_stride, (const bf16_t*)q, q_stride, (const bf16_t*)k_cache,
+        (const bf16_t*)v_cache, q_start, ctx_len, block_table, bt_stride, part_acc, part_ml, Hq, Hkv,
+        page_size, page_shift, window, keep_first, sink, scale * 1.4426950408889634f, num_splits);
+  else
+    attn_decode_mfma_kernel<NDT, UNR, false><<<grid, 256, lds, stream>>>(
+        (bf16_t*)out, out_stride, (const bf16_t*)q, q_stride, (const bf16_t*)k_cache,
+        (const bf16_t*)v_cache, q_start, ctx_len, block_table, bt_stride, part_acc, part_ml, Hq, Hkv,
+        page_size, page_shift, window, 0, sink, scale * 1.4426950408889634f, num_splits);
   if (hipGetLastError() != hipSuccess) return PTL_ERR_LAUNCH;
   if (num_splits > 1) {
     dim3 mgrid(n_seq, Hq);

@@ -65,8 +65,9 @@ template <> __device__ __forceinline__ void store4<float>(float* p, const float*
 }
 
 // NDK, NDV: key and value sizes in units of 32. RT: 16-row query tiles per wave; the workgroup
-// takes 64 * RT query rows.
-template <int NDK, int NDV, int RT, typename TO>
+// takes 64 * RT query rows. KEPT: a window that keeps the sequence's first keys (keep_first > 0):
+// the key tiles then walk a list of two stretches of positions instead of one.
+template <int NDK, int NDV, int RT, typename TO, bool KEPT>
 __global__ void __launch_bounds__(256, (NDK + NDV) <= 4 ? 3 : 2)
 attn_prefill_mfma_kernel(TO* __restrict__ out, long out_stride, const bf16_t* __restrict__ q,
                          long q_stride, const bf16_t* __restrict__ k_cache,
@@ -157,15 +158,27 @@ attn_prefill_mfma_kernel(TO* __restrict__ out, long out_stride, const bf16_t* __
   // and bfloat16 probabilities hold as well as values below 1, and nothing is rescaled
   const float lazy = 8.0f / scale_log2;
 
-  // The keys this block walks, as one list: the kept first keys left of the window (positions
-  // 0 .. n_kept - 1), then the positions from the window's start on. Tiles, k0 and the rows of a
-  // tile are indices of that list; key_at gives the position (the identity without a window).
-  const int k_lo = window > 0 ? max(0, first_q - window + 1) : 0;
-  const int n_kept = min(max(keep_first, 0), k_lo);
-  const int shift = k_lo - n_kept;
+  // The keys this block walks in tiles of 64, from index k_begin (a multiple of 64) on; indices
+  // below k_lo and from k_end on are no keys. Without kept keys an index is a position. KEPT: the
+  // list is the kept first keys left of the window (positions 0 .. n_kept - 1) and then the
+  // positions from the window's start on, index 0 is its first entry, and key_at gives the
+  // position of an index.
+  const int win_lo = window > 0 ? max(0, first_q - window + 1) : 0;
+  const int n_kept = KEPT ? min(max(keep_first, 0), win_lo) : 0;
+  const int shift = KEPT ? win_lo - n_kept : 0;
+  const int k_lo = KEPT ? 0 : win_lo;
   const int k_end = min(ctx, first_q + rows) - shift;
-  const int n_tiles = (k_end + PF_BN - 1) / PF_BN;
-  auto key_at = [&](int kw) { return kw < n_kept ? kw : kw + shift; };
+  const int k_begin = (k_lo / PF_BN) * PF_BN;
+  const int n_tiles = (k_end - k_begin + PF_BN - 1) / PF_BN;
+  auto key_at = [&](int kw) { return KEPT ? (kw < n_kept ? kw : kw + shift) : kw; };
+  // What a row sees, in indices: its own key is index qw; with kept keys, an index from n_kept on
+  // is a key of the window (position index + shift, which is no kept position when shift > 0),
+  // an index below is a kept key (a position below keep_first), so key_at is not needed there:
+  //   seen = kw <= qw && kw < k_end && (kw > qw - window || kw < keep_lim)
+  int qw[RT];
+#pragma unroll
+  for (int r = 0; r < RT; ++r) qw[r] = qpos[r] - shift;
+  const int keep_lim = shift == 0 ? keep_first : n_kept;
 
   // This thread's chunks of a tile. A wave's load instruction fills 64 consecutive 16-byte
   // slots of LDS, lane l the l-th; slot s holds row s / CPR, chunk (s % CPR) ^ swz(row).
@@ -192,11 +205,11 @@ attn_prefill_mfma_kernel(TO* __restrict__ out, long out_stride, const bf16_t* __
   const int page_mask = page_size - 1;                                // page sizes are powers of two
   // a tile that lies wholly inside the keys this block sees needs no tests (uniform)
   auto whole = [&](int t) {
-    const int k0 = t * PF_BN;
-    return t < n_tiles && k0 + PF_BN <= k_end;
+    const int k0 = k_begin + t * PF_BN;
+    return t < n_tiles && k0 >= k_lo && k0 + PF_BN <= k_end;
   };
   auto load_pages = [&](int t) {
-    const int k0 = t * PF_BN;
+    const int k0 = k_begin + t * PF_BN;
     if (whole(t)) {
 #pragma unroll
       for (int i = 0; i < NCHK; ++i) pgk[i] = bt[key_at(k0 + crowk[i]) >> page_shift];
@@ -207,13 +220,13 @@ attn_prefill_mfma_kernel(TO* __restrict__ out, long out_stride, const bf16_t* __
       for (int i = 0; i < NCHK; ++i) {
         const int kp = k0 + crowk[i];
         pgk[i] = -1;
-        if (t < n_tiles && kp < k_end) pgk[i] = bt[key_at(kp) >> page_shift];
+        if (t < n_tiles && kp >= k_lo && kp < k_end) pgk[i] = bt[key_at(kp) >> page_shift];
       }
 #pragma unroll
       for (int i = 0; i < NCHV; ++i) {
         const int kp = k0 + crowv[i];
         pgv[i] = -1;
-        if (t < n_tiles && kp < k_end) pgv[i] = bt[key_at(kp) >> page_shift];
+        if (t < n_tiles && kp >= k_lo && kp < k_end) pgv[i] = bt[key_at(kp) >> page_shift];
       }
     }
   };
@@ -225,7 +238,7 @@ attn_prefill_mfma_kernel(TO* __restrict__ out, long out_stride, const bf16_t* __
         (__attribute__((address_space(3))) void*)(tile_lds + 512 * chunk), 16, 0, 0);
   };
   auto fetch = [&](int t, bf16_t* Kb, bf16_t* Vb) {
-    const int k0 = t * PF_BN;
+    const int k0 = k_begin + t * PF_BN;
     const bool all = whole(t);
 #pragma unroll
     for (int i = 0; i < NCHK; ++i) {
@@ -287,9 +300,8 @@ attn_prefill_mfma_kernel(TO* __restrict__ out, long out_stride, const bf16_t* __
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
             const int kw = k0 + 16 * kt + 4 * lg + i;
-            const int key = key_at(kw);
-            const bool vis = key <= qpos[r] && kw < k_end &&
-                             (window <= 0 || key > qpos[r] - window || key < keep_first);
+            const bool vis = kw <= qw[r] && kw < k_end &&
+                             (window <= 0 || kw > qw[r] - window || (KEPT && kw < keep_lim));
             st[r][kt][i] = vis ? st[r][kt][i] : -INFINITY;
           }
       }
@@ -348,14 +360,14 @@ attn_prefill_mfma_kernel(TO* __restrict__ out, long out_stride, const bf16_t* __
   // one turn: tile t + 1 sets out for the other buffer (everyone left it before the last
   // barrier), tile t is used, and what was loaded is waited for before the barrier
   auto turn = [&](int t, bf16_t* Kb, bf16_t* Vb, bf16_t* Kn, bf16_t* Vn) {
-    const int k0 = t * PF_BN;
+    const int k0 = k_begin + t * PF_BN;
     if (t + 1 < n_tiles) {
       fetch(t + 1, Kn, Vn);
       load_pages(t + 2);
     }
     // a wave whose rows all lie before this tile has nothing to do in it
-    if (wave_has_rows && key_at(k0) <= wave_max_q) {
-      // (without a window an index of the walk is a position)
+    if (wave_has_rows && k0 <= wave_max_q - shift) {
+      // (without a window an index is a position)
       const bool need_mask = (k0 + PF_BN - 1 > wave_min_q) || (k0 + PF_BN > k_end) || window > 0;
       if (need_mask)
         tile(k0, Kb, Vb, std::true_type{});
@@ -407,11 +419,18 @@ static int launch_prefill_mfma(void* out, long out_stride, const void* q, long q
   int page_shift = -1;
   for (int sh = 0; sh < 31; ++sh)
     if ((1 << sh) == page_size) page_shift = sh;
-  attn_prefill_mfma_kernel<NDK, NDV, RT, TO><<<grid, 256, 0, stream>>>(
-      (TO*)out, out_stride, (const bf16_t*)q, q_stride, (const bf16_t*)k_cache,
-      (const bf16_t*)v_cache, q_start, ctx_len, block_table, bt_stride, work_seq, work_qoff,
-      n_work, Hq, Hkv, maps, page_size, page_shift, window, keep_first, sink,
-      scale * 1.4426950408889634f);
+  if (window > 0 && keep_first > 0)
+    attn_prefill_mfma_kernel<NDK, NDV, RT, TO, true><<<grid, 256, 0, stream>>>(
+        (TO*)out, out_stride, (const bf16_t*)q, q_stride, (const bf16_t*)k_cache,
+        (const bf16_t*)v_cache, q_start, ctx_len, block_table, bt_stride, work_seq, work_qoff,
+        n_work, Hq, Hkv, maps, page_size, page_shift, window, keep_first, sink,
+        scale * 1.4426950408889634f);
+  else
+    attn_prefill_mfma_kernel<NDK, NDV, RT, TO, false><<<grid, 256, 0, stream>>>(
+        (TO*)out, out_stride, (const bf16_t*)q, q_stride, (const bf16_t*)k_cache,
+        (const bf16_t*)v_cache, q_start, ctx_len, block_table, bt_stride, work_seq, work_qoff,
+        n_work, Hq, Hkv, maps, page_size, page_shift, window, 0, sink,
+        scale * 1.4426950408889634f);
   return ptl_launch_status();
 }
 
