@@ -50,10 +50,12 @@ __device__ __forceinline__ float unary_act(int kind, float u) {
   return r * r;
 }
 
-// One wave a token. Lane l holds the logits of experts l, l + 64, ...
-#define TOPK_PER_LANE 16
+// One wave a token. Lane l holds the logits of experts l, l + 64, ...: TOPK_PER_LANE of them
+// (1, 4 or 16, the least that covers the router's outputs).
+#define TOPK_MAX_PER_LANE 16
 #define SCORE_SIGMOID 0
 #define SCORE_SOFTMAX 1
+template <int TOPK_PER_LANE>
 __global__ void __launch_bounds__(256)
 moe_topk_kernel(const float* __restrict__ logits, int ld, int T_, int E, int top, int extra,
                 int renormalize, int score_fn, const float* __restrict__ bias, int real, float renorm_eps,
@@ -208,13 +210,18 @@ extern "C" int ptl_moe_topk(const float* logits, int ld, int T_, int E, int top,
   if (n_groups > 1 && (n_groups > 64 || E % n_groups || keep_groups < 1 || keep_groups > n_groups ||
                        (long)keep_groups * (E / n_groups) < top))
     return PTL_ERR_ARG;
-  if (E <= 0 || top <= 0 || top > E || E > 64 * TOPK_PER_LANE || extra < 0 || extra > 64 || ld < E + extra ||
+  if (E <= 0 || top <= 0 || top > E || E > 64 * TOPK_MAX_PER_LANE || extra < 0 || extra > 64 || ld < E + extra ||
       (extra && !extra_out) || real < 0 || real > E || (real < E && !ident_out) ||
       (score_fn != SCORE_SIGMOID && score_fn != SCORE_SOFTMAX))
     return PTL_ERR_ARG;
-  moe_topk_kernel<<<(T_ + 3) / 4, 256, 0, st>>>(logits, ld, T_, E, top, extra, renormalize, score_fn, bias, real,
-                                                renorm_eps, wscale, n_groups, keep_groups, idx, wgt,
-                                                extra_out, ident_out);
+#define GO(PER)                                                                                              \
+  moe_topk_kernel<PER><<<(T_ + 3) / 4, 256, 0, st>>>(logits, ld, T_, E, top, extra, renormalize, score_fn, bias, \
+                                                     real, renorm_eps, wscale, n_groups, keep_groups, idx, wgt,  \
+                                                     extra_out, ident_out)
+  if (E <= 64) GO(1);
+  else if (E <= 256) GO(4);
+  else GO(16);
+#undef GO
   return ptl_launch_status();
 }
 
