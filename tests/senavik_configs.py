@@ -5,8 +5,8 @@ exactly a page, more than a page, more than the window); rotations of a whole he
 none, with and without rescaled frequencies, with band edges and ramps that meet all their
 branches (also a ramp whose ends coincide); one to four heads a kv head; key and value sizes that
 are equal, that differ either way and that are no multiple of 16; latents whose size with the
-rotated part is 24, 32, 40, 64 and 96 (so the vector, split-KV and matrix-core kernels are all
-met); query latents smaller and larger than the width; dense, routed and absent feed-forwards;
+rotated part is 24, 32, 40, 64, 96 and 128 under 1 to 20 heads (so the vector, split-KV and
+matrix-core kernels are all met); query latents smaller and larger than the width; dense, routed and absent feed-forwards;
 experts in 1 to 6 groups of 1 to 4 of which 1 to all are kept, and no groups entry; 1 to 3
 experts a token."""
 import copy
@@ -116,9 +116,23 @@ def _s5():
     ])
 
 
+def _s6():
+    """Pages of 16. Head sizes of real models: attention with keys and values of 128, four heads a kv
+    head, half a head rotating, a window of 64 that keeps 4; latents of 96 + 32 = 128 under 16 heads
+    (the most the matrix-core decode kernel takes on one kv head) and under 20 (the vector split-KV
+    kernel); 16 experts in 4 groups of which 2 are kept."""
+    return model(300, 128, 1e-6, [
+        layer(attention(8, 2, 128, 128, 0.09, window=64, keep_first=4, rot=(500000.0, 64), scaling=(8.0, 1.0, 4.0, 256)),
+              dense(160)),
+        layer(latent(16, 64, 32, 64, 96, 96, 0.1, rot=(10000.0, 32), scaling=(40.0, 128, 32.0, 1.0)),
+              moe(64, 16, 2, groups=(4, 2))),
+        layer(latent(20, 32, 32, 32, 96, 48, 0.12, rot=(10000.0, 32)), None),
+    ])
+
+
 # name -> (config, weight std, page size)
 SENAVIK = {"S1": (_s1(), 0.12, 4), "S2": (_s2(), 0.15, 8), "S3": (_s3(), 0.12, 16), "S4": (_s4(), 0.12, 8),
-           "S5": (_s5(), 0.15, 4)}
+           "S5": (_s5(), 0.15, 4), "S6": (_s6(), 0.08, 16)}
 
 
 def senavik(name):

@@ -22,9 +22,9 @@ pytestmark = pytest.mark.gpu
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 LENGTHS = {"S1": [5, 9, 33, 70, 130, 47], "S2": [3, 17, 40, 65, 31], "S3": [12, 50, 90, 20, 2, 150],
-           "S4": [7, 30, 64, 81, 120], "S5": [9, 44, 66, 1]}
+           "S4": [7, 30, 64, 81, 120], "S5": [9, 44, 66, 1], "S6": [150, 21, 77]}
 DTYPES = [torch.float32, torch.bfloat16]
-NAMES = ["S1", "S2", "S3", "S4", "S5"]
+NAMES = ["S1", "S2", "S3", "S4", "S5", "S6"]
 ROUTER_GAIN = 2.0       # routers this much larger than the other matrices (more would saturate the sigmoid)
 
 
@@ -338,7 +338,7 @@ def test_pages_behind_a_window_are_given_back_and_the_kept_ones_stay(cases):
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=["fp32", "bf16"])
-@pytest.mark.parametrize("name", ["S1", "S3", "S5"])
+@pytest.mark.parametrize("name", ["S1", "S3", "S5", "S6"])
 def test_cuttings_replayed_as_graphs(cases, name, dtype):
     """Decode steps and single portions replayed as HIP graphs (padded layouts: rows that belong
     to nobody) against the plain model."""
