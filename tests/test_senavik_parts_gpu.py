@@ -290,7 +290,6 @@ def test_latent_preparation_in_the_half_layout(gpu_device, dtype, H, dn, dr, R, 
 @pytest.mark.parametrize("name", ["latent", "attention"])
 def test_mixers_as_parts_over_a_fresh_cache(gpu_device, dtype, name):
     """One mixer alone, a whole prompt, against the plain function."""
-    from engine_helpers import load_runner  # noqa: F401  (registers nothing; keeps imports alike)
     from pytriton_llama_amd.cache import CacheManager, CacheStorage
     from pytriton_llama_amd.engine.batch import StepEntry, build_context
     from pytriton_llama_amd.parts import build_part
