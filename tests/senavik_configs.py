@@ -138,3 +138,53 @@ SENAVIK = {"S1": (_s1(), 0.12, 4), "S2": (_s2(), 0.15, 8), "S3": (_s3(), 0.12, 1
 def senavik(name):
     cfg, std, page = SENAVIK[name]
     return copy.deepcopy(cfg), std, page
+
+
+def drawn(seed):
+    """A configuration drawn from the ranges a model of this design may lie in (pages of 16):
+    2 to 5 layers of either kind in any order, head sizes 16 to 128, 1 to 4 heads a kv head,
+    windows from 8 to 130 or none with 0 to 20 kept tokens, rotations of none, part or all of a
+    head with or without rescaled frequencies, latents of 40 to 128 with the rotated part, dense,
+    routed or absent feed-forwards with 4 to 32 experts in groups."""
+    import random
+    rng = random.Random(seed)
+    width = rng.choice([64, 96, 128, 192, 256])
+    layers = []
+    for _ in range(rng.randint(2, 5)):
+        if rng.random() < 0.55:
+            kv = rng.choice([1, 2, 4])
+            dim, vdim = rng.choice([16, 32, 48, 64, 96, 128]), rng.choice([16, 32, 48, 64, 96, 128])
+            if rng.random() < 0.5:
+                vdim = dim
+            window = rng.choice([None, 8, 33, 64, 96, 130])
+            keep = rng.choice([None, 0, 1, 4, 16, 20]) if window else None
+            rot = None
+            if rng.random() < 0.85:
+                rot = (rng.choice([10000.0, 20000.0, 500000.0]), rng.choice([dim, dim // 2, 8]))
+            scaling = (rng.choice([2.0, 8.0]), 1.0, rng.choice([2.0, 4.0]), rng.choice([32, 64, 256])) \
+                if rot and rng.random() < 0.7 else None
+            mixer = attention(kv * rng.choice([1, 2, 4]), kv, dim, vdim, rng.uniform(0.7, 1.3) * dim ** -0.5,
+                              window=window, keep_first=keep, rot=rot, scaling=scaling)
+        else:
+            dim, rot_dim = rng.choice([16, 32, 64]), rng.choice([8, 16, 32])
+            kv_rank = rng.choice([32, 48, 64, 96])
+            scaling = (rng.choice([4.0, 40.0]), rng.choice([32, 128]), rng.choice([8.0, 32.0]), rng.choice([1.0, 2.0])) \
+                if rng.random() < 0.7 else None
+            mixer = latent(rng.choice([2, 4, 6, 8, 16]), dim, rot_dim, rng.choice([16, 32, 64, 80]), kv_rank,
+                           rng.choice([32, 64, 128]), rng.uniform(0.7, 1.3) * (dim + rot_dim) ** -0.5,
+                           rot=(rng.choice([10000.0, 250000.0]), rot_dim), scaling=scaling)
+        kind = rng.random()
+        if kind < 0.2:
+            mlp = None
+        elif kind < 0.45:
+            mlp = dense(rng.choice([64, 96, 256]))
+        else:
+            experts = rng.choice([4, 8, 16, 32])
+            count = rng.choice([c for c in (1, 2, 4, 8) if experts % c == 0])
+            keep_groups = rng.randint(1, count)
+            top = rng.randint(1, min(4, keep_groups * (experts // count)))
+            mlp = moe(rng.choice([32, 64, 96]), experts, top, groups=(count, keep_groups) if rng.random() < 0.85 else None)
+            if mlp["router"].get("groups") is None:
+                mlp = moe(mlp["expert"]["ff"], experts, min(top, experts))
+        layers.append(layer(mixer, mlp))
+    return model(rng.randint(100, 600), width, rng.choice([1e-6, 1e-5]), layers), 0.1, 16

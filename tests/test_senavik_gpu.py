@@ -358,6 +358,25 @@ def test_cuttings_replayed_as_graphs(cases, name, dtype):
         assert bad is None, f"{name} {dtype}: {bad}"
 
 
+@pytest.mark.parametrize("seed", range(12))
+def test_drawn_configurations(tmp_path_factory, gpu_device, seed):
+    """Configurations drawn at random from the ranges of the design, pages of 16: whole prompts,
+    the last tokens one by one, and mixed batches on few pages, in both precisions."""
+    from senavik_configs import drawn
+    cfg, std, page = drawn(seed)
+    folder, _ = write_folder(tmp_path_factory, "S1", seed=200 + seed, cfg=cfg)
+    seqs = random_sequences(cfg["vocab"], [190, 45, 3, 101], seed=seed)
+    touchy = {}
+    want = {torch.float32: plain_logits(folder, seqs), torch.bfloat16: plain_logits(folder, seqs, torch.bfloat16, touchy),
+            "touchy": touchy}
+    cases = {"D": (folder, page, seqs, want)}
+    for dtype in DTYPES:
+        run_cutting(cases, "D", dtype, cuttings.tail_decode(seqs, 36))
+        steps = cuttings.mixed(seqs, seed=seed, max_live=3)
+        run_cutting(cases, "D", dtype, steps, cuttings.max_live_tokens(steps, round_to=page) // page, max_num_seqs=3)
+    run_cutting(cases, "D", torch.float32, cuttings.portions(seqs))
+
+
 def plain_greedy(folder, prompt, n):
     cfg, w = read_folder(folder)
     toks = list(prompt)
